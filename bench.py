@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Benchmark of the HSTU attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--tile-config ID] [--no-cpu]
+
+A step is one forward pass (one launch) over one synthetic jagged batch that is already resident in
+HBM.  Prints ONE JSON line: the headline metric, the MFMA (or HBM) roofline of the kernel computed
+from algorithmic work and HIP-event time, and the CPU oracle timed on a bounded sample of the same
+workload on this box's host cores.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
+PEAK_HBM_GBS = 8000.0
+HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced against HBM bandwidth
+
+
+def run_gpu(wl, args, pkg, workloads, torch):
+    dev = torch.device("cuda:0")
+    inp = workloads.make_inputs(wl, dev, fused_buffer=args.fused_buffer)
+    q, k, v = inp["q"], inp["k"], inp["v"]
+    kw = dict(num_targets=inp["num_targets"], max_attn_len=wl.max_attn_len, contextual_seq_len=wl.contextual_seq_len,
+              tile_config=args.tile_config)
+    scales = {}
+    if wl.dtype == "fp8":
+        qs, ks, vs = [float(x.float().abs().max()) / 448.0 for x in (q, k, v)]
+        q = (q.float() / qs).to(torch.float8_e4m3fn)
+        k = (k.float() / ks).to(torch.float8_e4m3fn)
+        v = (v.float() / vs).to(torch.float8_e4m3fn)
+        scales = dict(q_scale=qs, k_scale=ks, v_scale=vs)
+    if wl.delta_size > 0:
+        def step():
+            return pkg.delta_hstu_mha(wl.max_seq_len, wl.alpha, q, k, v, inp["seq_offsets"], **kw, **scales)
+    else:
+        def step():
+            return pkg.hstu_mha(wl.max_seq_len, wl.alpha, q, k, v, inp["seq_offsets"],
+                                min_full_attn_seq_len=wl.min_full_attn_seq_len, **kw, **scales)
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    # HIP events on the stream the kernel is launched on (torch's current stream).
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        out = step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = start.elapsed_time(stop) / args.steps
+    del out
+    return wall_ms, ev_ms
+
+
+def run_cpu_baseline(wl, torch, workloads, budget_s=20.0):
+    """The PyTorch oracle (per-sequence form of the reference's pytorch_hstu_mha, fp32) on a bounded sample."""
+    from oracle import hstu_oracle
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    inp = workloads.make_inputs(wl, torch.device("cpu"), dtype=torch.float32)
+    order = sorted(range(wl.batch), key=lambda b: -int(wl.lengths[b]))
+    # sample: the longest sequence first, then every 8th by length, until the time budget is spent
+    picks = [order[0]] + order[8::8]
+    done, flops, t_used = [], 0.0, 0.0
+    for b in picks:
+        sub = workloads.Workload(
+            "s", 1, wl.heads, wl.dqk, wl.dv, wl.max_seq_len, wl.lengths[b : b + 1],
+            None if wl.num_targets is None else wl.num_targets[b : b + 1], wl.max_attn_len,
+            wl.contextual_seq_len, wl.min_full_attn_seq_len, wl.delta_size, wl.dtype, wl.alpha,
+        )
+        t0 = time.perf_counter()
+        hstu_oracle.hstu_mha_per_sequence(
+            wl.max_seq_len, wl.alpha, inp["q"], inp["k"], inp["v"], inp["seq_offsets"], num_targets=inp["num_targets"],
+            max_attn_len=wl.max_attn_len, contextual_seq_len=wl.contextual_seq_len,
+            min_full_attn_seq_len=wl.min_full_attn_seq_len, delta_size=wl.delta_size, sequences=[b],
+        )
+        t_used += time.perf_counter() - t0
+        flops += workloads.algorithmic_flops(sub)
+        done.append(b)
+        if t_used > budget_s:
+            break
+    return {
+        "value": round(flops / t_used / 1e12, 5),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{len(done)} of {wl.batch} sequences of workload {wl.name} (lengths "
+        f"{[int(wl.lengths[b]) for b in done]}), fp32 PyTorch oracle per sequence, {t_used:.1f} s",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="headline")
+    ap.add_argument("--tile-config", type=int, default=0)
+    ap.add_argument("--fused-buffer", action="store_true", help="q/k/v as column slices of one [L,H,3D] buffer")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
+              "(sequences are independent, so N GPUs would each run the same kernel on a slice)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import __graft_entry__
+
+    pkg = __graft_entry__.load_package()
+    from generative_recommenders_amd import workloads
+
+    wl = workloads.make_workload(args.workload)
+    if wl.dtype == "fp32":
+        print("bench.py: cfg1 is the CPU correctness case, not a GPU bench workload", file=sys.stderr)
+        sys.exit(2)
+    wall_ms, ev_ms = run_gpu(wl, args, pkg, workloads, torch)
+    flops = workloads.algorithmic_flops(wl)
+    ref_flops = workloads.reference_convention_flops(wl)
+    nbytes = workloads.algorithmic_bytes(wl)
+    tflops = flops / (ev_ms * 1e-3) / 1e12
+    if wl.name in HBM_BOUND:
+        ach = nbytes / (ev_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
+    else:
+        peak = PEAK_TFLOPS[wl.dtype]
+        roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(tflops / peak, 4), "traffic": None}
+    roof["kernel"] = "hstu_fwd_kernel"
+    roof["kernel_ms"] = round(ev_ms, 4)
+    roof["algorithmic_flops"] = flops
+    roof["algorithmic_bytes"] = nbytes
+    line = {
+        "metric": "HSTU attn fwd effective TFLOP/s + % MFMA peak, jagged B=64 L<=8192 H4 d128",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": wl.dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": wl.name,
+            "batch": wl.batch, "heads": wl.heads, "dqk": wl.dqk, "dv": wl.dv, "max_seq_len": wl.max_seq_len,
+            "total_tokens": wl.total_kv, "max_attn_len": wl.max_attn_len, "contextual_seq_len": wl.contextual_seq_len,
+            "num_targets": wl.num_targets is not None, "delta_size": wl.delta_size,
+            "tile_config": args.tile_config, "fused_buffer": args.fused_buffer,
+        },
+        "pct_mfma_peak": round(100.0 * tflops / PEAK_TFLOPS[wl.dtype], 2),
+        "reference_convention_tflops": round(ref_flops / (ev_ms * 1e-3) / 1e12, 2),
+        "hbm_gbs_algorithmic": round(nbytes / (ev_ms * 1e-3) / 1e9, 1),
+        "roofline": roof,
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = run_cpu_baseline(wl, torch, workloads)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

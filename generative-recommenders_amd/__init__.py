@@ -1,0 +1,12 @@
+"""MI355X-native HSTU jagged attention (forward): ``hstu_mha`` and ``delta_hstu_mha``.
+
+Drop-in for ``generative_recommenders.ops.hstu_attention`` of the reference, backed by
+hand-written gfx950 HIP kernels behind a C ABI (``csrc/``, ``include/hstu_hip.h``).
+The directory name contains a hyphen, so load it with ``importlib`` under the module name
+``generative_recommenders_amd`` (``__graft_entry__.load_package()`` does exactly that).
+"""
+
+from .common import HammerKernel  # noqa: F401
+from .ops.hstu_attention import delta_hstu_mha, hstu_mha  # noqa: F401
+
+__all__ = ["HammerKernel", "hstu_mha", "delta_hstu_mha"]

@@ -1,0 +1,181 @@
+// C ABI of libhstu_hip.so: argument validation, kernel selection and launch.
+// Declarations and the reference interfaces they replace are in include/hstu_hip.h.
+#include "hstu_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "hstu_fwd_kernel.h"
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+void set_last_error(const char* what, hipError_t e) {
+    snprintf(g_last_error, sizeof(g_last_error), "%s: %s", what, hipGetErrorString(e));
+}
+
+struct TileConfig {
+    const char* name;
+    int qt, nw, bn;  // query tiles (of 32 rows) per wave, waves per workgroup, kv rows per tile
+};
+// id 1..: see hstu_hip_tile_configs()
+const TileConfig kConfigs[] = {
+    {"m128n64w4", 1, 4, 64},
+    {"m256n64w4", 2, 4, 64},
+};
+constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
+
+template <class TT, int DQK, int DV, int QT, int NW, int BN, int OCC>
+int launch(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
+    constexpr int BM = NW * QT * 32;
+    constexpr int smem = 2 * BN * (DQK + DV) * 2;
+    auto kern = hstu::hstu_fwd_kernel<TT, DQK, DV, QT, NW, BN, OCC>;
+    static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; racing threads set the same value
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) {
+            set_last_error("hipFuncSetAttribute", e);
+            return HSTU_ERR_LAUNCH;
+        }
+        attr_done = true;
+    }
+    (void)BM;
+    const int pairs_per_xcd = (num_pairs + 7) / 8;
+    const long long grid = (long long)pairs_per_xcd * 8 * p.num_mb;
+    if (grid <= 0) return HSTU_OK;
+    if (grid > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), smem, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_last_error("kernel launch", e);
+        return HSTU_ERR_LAUNCH;
+    }
+    return HSTU_OK;
+}
+
+template <class TT, int D>
+int launch_cfg(const hstu::FwdParams& p0, int cfg, int rows_per_pair, int num_pairs, hipStream_t stream) {
+    hstu::FwdParams p = p0;
+    if (cfg == 2) {
+        p.num_mb = (rows_per_pair + 255) / 256;
+        return launch<TT, D, D, 2, 4, 64, 1>(p, num_pairs, stream);
+    }
+    p.num_mb = (rows_per_pair + 127) / 128;
+    return launch<TT, D, D, 1, 4, 64, 2>(p, num_pairs, stream);
+}
+
+template <class TT>
+int launch_dim(const hstu::FwdParams& p, int d, int cfg, int rows_per_pair, int num_pairs, hipStream_t stream) {
+    switch (d) {
+        case 32: return launch_cfg<TT, 32>(p, cfg, rows_per_pair, num_pairs, stream);
+        case 64: return launch_cfg<TT, 64>(p, cfg, rows_per_pair, num_pairs, stream);
+        case 128: return launch_cfg<TT, 128>(p, cfg, rows_per_pair, num_pairs, stream);
+        default: return HSTU_ERR_BAD_HEAD_DIM;
+    }
+}
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int hstu_hip_version(void) { return 100; }
+
+const char* hstu_hip_status_string(int status) {
+    switch (status) {
+        case HSTU_OK: return "ok";
+        case HSTU_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case HSTU_ERR_BAD_DTYPE: return "only bf16, fp16 and fp8_e4m3 data types are supported";
+        case HSTU_ERR_BAD_HEAD_DIM: return "unsupported head dimension (built: dqk == dv in {32, 64, 128})";
+        case HSTU_ERR_MISALIGNED:
+            return "q/k/v/out must be 16-byte aligned with row and head strides that are multiples of 8 elements";
+        case HSTU_ERR_BAD_SHAPE: return "inconsistent sizes";
+        case HSTU_ERR_UNSUPPORTED: return "argument combination not built";
+        case HSTU_ERR_LAUNCH: return "HIP launch failed";
+        case HSTU_ERR_BAD_DEVICE: return "current device is not gfx950";
+        default: return "unknown status";
+    }
+}
+
+const char* hstu_hip_last_error(void) { return g_last_error; }
+
+int hstu_hip_tile_configs(void) { return kNumConfigs; }
+
+const char* hstu_hip_tile_config_name(int id) {
+    if (id < 1 || id > kNumConfigs) return "";
+    return kConfigs[id - 1].name;
+}
+
+int hstu_hip_check_args(const HstuFwdArgs* a) {
+    if (!a) return HSTU_ERR_NULL_POINTER;
+    if (a->dtype != HSTU_BF16 && a->dtype != HSTU_FP16 && a->dtype != HSTU_FP8_E4M3) return HSTU_ERR_BAD_DTYPE;
+    if (a->batch < 0 || a->heads <= 0 || a->total_q < 0 || a->total_kv < 0 || a->max_seq_len <= 0 ||
+        a->delta_size < 0 || a->max_attn_len < 0 || a->contextual_seq_len < 0 || a->min_full_attn_seq_len < 0)
+        return HSTU_ERR_BAD_SHAPE;
+    if (a->delta_size > 0 && a->total_q != (int64_t)a->batch * a->delta_size) return HSTU_ERR_BAD_SHAPE;
+    if (a->delta_size == 0 && a->total_q != a->total_kv) return HSTU_ERR_BAD_SHAPE;
+    if (a->total_kv > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    if (a->tile_config < 0 || a->tile_config > kNumConfigs) return HSTU_ERR_BAD_SHAPE;
+    if (a->dqk != a->dv) return HSTU_ERR_BAD_HEAD_DIM;  // as the reference's native op, flash_common.cpp:543-545
+    if (a->dqk != 32 && a->dqk != 64 && a->dqk != 128) return HSTU_ERR_BAD_HEAD_DIM;
+    if (a->total_q == 0 || a->batch == 0) return HSTU_OK;  // nothing to do; pointers may be anything
+    if (!a->q || !a->k || !a->v || !a->out || !a->seq_offsets) return HSTU_ERR_NULL_POINTER;
+    if (a->dtype == HSTU_FP8_E4M3) return HSTU_ERR_UNSUPPORTED;
+    if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out)) return HSTU_ERR_MISALIGNED;
+    const int64_t strides[8] = {a->q_row_stride, a->q_head_stride, a->k_row_stride, a->k_head_stride,
+                                a->v_row_stride, a->v_head_stride, a->o_row_stride, a->o_head_stride};
+    for (int i = 0; i < 8; ++i)
+        if (strides[i] < 0 || (strides[i] & 7) != 0) return HSTU_ERR_MISALIGNED;
+    return HSTU_OK;
+}
+
+int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
+    g_last_error[0] = 0;
+    int rc = hstu_hip_check_args(a);
+    if (rc != HSTU_OK) return rc;
+    if (a->total_q == 0 || a->batch == 0) return HSTU_OK;
+    hipStream_t stream = (hipStream_t)stream_;
+
+    hstu::FwdParams p;
+    memset(&p, 0, sizeof(p));
+    p.q = (const char*)a->q;
+    p.k = (const char*)a->k;
+    p.v = (const char*)a->v;
+    p.o = (char*)a->out;
+    p.q_rs = a->q_row_stride;
+    p.q_hs = a->q_head_stride;
+    p.k_rs = a->k_row_stride;
+    p.k_hs = a->k_head_stride;
+    p.v_rs = a->v_row_stride;
+    p.v_hs = a->v_head_stride;
+    p.o_rs = a->o_row_stride;
+    p.o_hs = a->o_head_stride;
+    p.offsets = a->seq_offsets;
+    p.targets = a->num_targets;
+    p.offsets_i64 = a->seq_offsets_i64;
+    p.targets_i64 = a->num_targets_i64;
+    p.B = a->batch;
+    p.H = a->heads;
+    p.max_seq_len = a->max_seq_len;
+    p.delta = a->delta_size;
+    p.w = a->max_attn_len;
+    p.c = a->contextual_seq_len;
+    p.f = a->min_full_attn_seq_len;
+    p.c1 = -a->alpha * 1.4426950408889634f;
+    p.oscale = a->alpha / (float)a->max_seq_len;
+
+    const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
+    const long long num_pairs_ll = (long long)a->batch * a->heads;
+    if (num_pairs_ll > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    const int num_pairs = (int)num_pairs_ll;
+    int cfg = a->tile_config;
+    if (cfg == 0) cfg = 1;
+    if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
+    return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,185 @@
+"""ctypes binding of ``libhstu_hip.so`` (C ABI declared in ``include/hstu_hip.h``)."""
+
+import ctypes
+import os
+from typing import Optional
+
+import torch
+
+from ..build import LIB_PATH
+
+HSTU_BF16, HSTU_FP16, HSTU_FP8_E4M3 = 0, 1, 2
+
+
+class HstuFwdArgs(ctypes.Structure):
+    """Field-for-field mirror of ``struct HstuFwdArgs``."""
+
+    _fields_ = [
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("q_row_stride", ctypes.c_int64),
+        ("q_head_stride", ctypes.c_int64),
+        ("k_row_stride", ctypes.c_int64),
+        ("k_head_stride", ctypes.c_int64),
+        ("v_row_stride", ctypes.c_int64),
+        ("v_head_stride", ctypes.c_int64),
+        ("o_row_stride", ctypes.c_int64),
+        ("o_head_stride", ctypes.c_int64),
+        ("seq_offsets", ctypes.c_void_p),
+        ("num_targets", ctypes.c_void_p),
+        ("seq_offsets_i64", ctypes.c_int32),
+        ("num_targets_i64", ctypes.c_int32),
+        ("batch", ctypes.c_int32),
+        ("heads", ctypes.c_int32),
+        ("dqk", ctypes.c_int32),
+        ("dv", ctypes.c_int32),
+        ("total_q", ctypes.c_int64),
+        ("total_kv", ctypes.c_int64),
+        ("max_seq_len", ctypes.c_int32),
+        ("delta_size", ctypes.c_int32),
+        ("alpha", ctypes.c_float),
+        ("max_attn_len", ctypes.c_int32),
+        ("contextual_seq_len", ctypes.c_int32),
+        ("min_full_attn_seq_len", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("q_scale", ctypes.c_float),
+        ("k_scale", ctypes.c_float),
+        ("v_scale", ctypes.c_float),
+        ("tile_config", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+EXPORTS = (
+    "hstu_hip_version",
+    "hstu_hip_status_string",
+    "hstu_hip_last_error",
+    "hstu_hip_check_args",
+    "hstu_hip_mha_fwd",
+    "hstu_hip_tile_configs",
+    "hstu_hip_tile_config_name",
+)
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def library_path() -> str:
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library.  Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
+                "(hipcc --offload-arch=gfx950).  There is no CPU or PyTorch fallback."
+            )
+        L = ctypes.CDLL(LIB_PATH)
+        L.hstu_hip_version.restype = ctypes.c_int
+        L.hstu_hip_status_string.restype = ctypes.c_char_p
+        L.hstu_hip_status_string.argtypes = [ctypes.c_int]
+        L.hstu_hip_last_error.restype = ctypes.c_char_p
+        L.hstu_hip_check_args.restype = ctypes.c_int
+        L.hstu_hip_check_args.argtypes = [ctypes.POINTER(HstuFwdArgs)]
+        L.hstu_hip_mha_fwd.restype = ctypes.c_int
+        L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
+        L.hstu_hip_tile_configs.restype = ctypes.c_int
+        L.hstu_hip_tile_config_name.restype = ctypes.c_char_p
+        L.hstu_hip_tile_config_name.argtypes = [ctypes.c_int]
+        _lib = L
+    return _lib
+
+
+_STATUS_EXC = {
+    -1: ValueError,
+    -2: RuntimeError,  # the reference raises RuntimeError via TORCH_CHECK for dtype / layout problems
+    -3: RuntimeError,
+    -4: RuntimeError,
+    -5: ValueError,
+    -6: NotImplementedError,
+    -7: RuntimeError,
+    -8: RuntimeError,
+}
+
+
+def raise_for_status(rc: int) -> None:
+    if rc == 0:
+        return
+    L = lib()
+    msg = L.hstu_hip_status_string(rc).decode()
+    extra = L.hstu_hip_last_error().decode()
+    if extra:
+        msg = f"{msg} ({extra})"
+    raise _STATUS_EXC.get(rc, RuntimeError)(f"hstu_hip: {msg} [status {rc}]")
+
+
+def tile_config_names() -> list:
+    L = lib()
+    return [L.hstu_hip_tile_config_name(i + 1).decode() for i in range(L.hstu_hip_tile_configs())]
+
+
+def _dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.bfloat16:
+        return HSTU_BF16
+    if dt == torch.float16:
+        return HSTU_FP16
+    if dt == torch.float8_e4m3fn:
+        return HSTU_FP8_E4M3
+    raise RuntimeError(f"hstu_hip only supports fp16, bf16, and fp8_e4m3 data type, got {dt}")
+
+
+def mha_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    seq_offsets: torch.Tensor,
+    num_targets: Optional[torch.Tensor],
+    max_seq_len: int,
+    alpha: float,
+    delta_size: int,
+    max_attn_len: int,
+    contextual_seq_len: int,
+    min_full_attn_seq_len: int,
+    q_scale: float = 1.0,
+    k_scale: float = 1.0,
+    v_scale: float = 1.0,
+    tile_config: int = 0,
+) -> None:
+    """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors."""
+    a = HstuFwdArgs()
+    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
+    a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
+    a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
+    a.o_row_stride, a.o_head_stride = out.stride(0), out.stride(1)
+    a.seq_offsets = seq_offsets.data_ptr()
+    a.seq_offsets_i64 = 1 if seq_offsets.dtype == torch.int64 else 0
+    if num_targets is not None:
+        a.num_targets = num_targets.data_ptr()
+        a.num_targets_i64 = 1 if num_targets.dtype == torch.int64 else 0
+    else:
+        a.num_targets = None
+    a.batch = seq_offsets.numel() - 1
+    a.heads = q.shape[1]
+    a.dqk = q.shape[2]
+    a.dv = v.shape[2]
+    a.total_q = q.shape[0]
+    a.total_kv = k.shape[0]
+    a.max_seq_len = max_seq_len
+    a.delta_size = delta_size
+    a.alpha = alpha
+    a.max_attn_len = max_attn_len
+    a.contextual_seq_len = contextual_seq_len
+    a.min_full_attn_seq_len = min_full_attn_seq_len
+    a.dtype = _dtype_code(q.dtype)
+    a.q_scale, a.k_scale, a.v_scale = q_scale, k_scale, v_scale
+    a.tile_config = tile_config
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        rc = lib().hstu_hip_mha_fwd(ctypes.byref(a), ctypes.c_void_p(stream))
+    raise_for_status(rc)

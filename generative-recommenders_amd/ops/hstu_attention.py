@@ -1,0 +1,198 @@
+"""``hstu_mha`` / ``delta_hstu_mha`` with the reference's signatures, running on gfx950 HIP kernels.
+
+Mirrors ``generative_recommenders/ops/hstu_attention.py`` of the reference (``hstu_mha``
+at lines 101-207, ``delta_hstu_mha`` at lines 210-284): same argument names, defaults, assertion
+messages and output shapes.  Differences, all explicit:
+
+* there is one backend, so ``kernel`` / ``enable_tma`` / ``sort_by_length`` are accepted and ignored;
+* forward only -- inputs that require grad under ``torch.enable_grad()`` raise ``NotImplementedError``;
+* tensors must live on a HIP device; there is no CPU or PyTorch fallback;
+* fp8 (``torch.float8_e4m3fn``) q/k/v take per-tensor scales through ``q_scale``/``k_scale``/``v_scale``
+  and give bf16 output, as the reference's native op does (``flash_common.cpp:596-607``).
+"""
+
+from typing import Optional
+
+import torch
+
+from ..common import HammerKernel, switch_to_contiguous_if_needed
+from . import hip_backend
+
+
+def _kernel_layout(x: torch.Tensor) -> torch.Tensor:
+    """Dense innermost dim (``common.py:262-269``) and 16-byte aligned rows, copying only if needed."""
+    x = switch_to_contiguous_if_needed(x)
+    per16 = 16 // x.element_size()
+    if x.data_ptr() % 16 != 0 or x.stride(0) % per16 != 0 or x.stride(1) % per16 != 0:
+        x = x.contiguous()
+        if x.data_ptr() % 16 != 0:
+            x = x.clone(memory_format=torch.contiguous_format)
+    return x
+
+
+def _index_tensor(x: torch.Tensor, name: str) -> torch.Tensor:
+    torch._assert(x.dtype in (torch.int32, torch.int64), f"{name} must be int32 or int64")
+    return x.contiguous()
+
+
+def _check_forward_only(*tensors: torch.Tensor) -> None:
+    if torch.is_grad_enabled() and any(t.requires_grad for t in tensors):
+        raise NotImplementedError(
+            "the HIP backend implements the forward pass only; call it under torch.no_grad() "
+            "or detach the inputs"
+        )
+
+
+def _require_device(t: torch.Tensor, name: str) -> None:
+    # same wording as hstu_attention.py:132-135 of the reference
+    torch._assert(t.is_cuda, f"{name} must be CUDA tensor")
+
+
+def hstu_mha(
+    max_seq_len: int,
+    alpha: float,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    seq_offsets: torch.Tensor,
+    causal: bool = True,
+    dropout_pr: float = 0.0,
+    training: bool = True,
+    num_targets: Optional[torch.Tensor] = None,
+    attn_scale: Optional[torch.Tensor] = None,
+    max_attn_len: int = 0,
+    contextual_seq_len: int = 0,
+    min_full_attn_seq_len: int = 0,
+    sort_by_length: bool = False,
+    kernel: HammerKernel = HammerKernel.HIP,
+    enable_tma: bool = False,
+    q_scale: float = 1.0,
+    k_scale: float = 1.0,
+    v_scale: float = 1.0,
+    tile_config: int = 0,
+) -> torch.Tensor:
+    """Jagged HSTU attention forward; returns ``[L, H, Dv]``.
+
+    ``out[r] = sum_s M(r, s) * silu(alpha * q_r . k_s) / max_seq_len * v_s`` per sequence and head.
+    """
+    torch._assert(max_seq_len > 0, "max_seq_len must be larger than 0")
+    torch._assert(q.dim() == 3, "q must be 3-D")
+    torch._assert(k.shape == q.shape, "k must be the same shape as q")
+    torch._assert(v.dim() == 3, "v must be 3-D")
+    torch._assert(v.shape[0] == q.shape[0], "wrong v shape[0]")
+    torch._assert(v.shape[1] == q.shape[1], "wrong v shape[1]")
+    torch._assert(causal, "only support causal attention")
+    _require_device(q, "q")
+    _require_device(k, "k")
+    _require_device(v, "v")
+    _require_device(seq_offsets, "seq_offsets")
+    torch._assert(dropout_pr < 1e-6, "dropout for triton path not implemented")
+    assert attn_scale is None, "attn_scale not implemented"
+    torch._assert(k.dtype == q.dtype and v.dtype == q.dtype, "q, k and v must have the same dtype")
+    if num_targets is not None:
+        _require_device(num_targets, "num_targets")
+        torch._assert(num_targets.numel() == seq_offsets.numel() - 1, "num_targets must have one entry per sequence")
+        num_targets = _index_tensor(num_targets, "num_targets")
+    _check_forward_only(q, k, v)
+    seq_offsets = _index_tensor(seq_offsets, "seq_offsets")
+
+    q = _kernel_layout(q.detach())
+    k = _kernel_layout(k.detach())
+    v = _kernel_layout(v.detach())
+    out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else v.dtype
+    out = torch.empty((v.shape[0], v.shape[1], v.shape[2]), dtype=out_dtype, device=v.device)
+    if out.numel() == 0:
+        return out
+    hip_backend.mha_fwd(
+        q,
+        k,
+        v,
+        out,
+        seq_offsets,
+        num_targets,
+        max_seq_len=max_seq_len,
+        alpha=alpha,
+        delta_size=0,
+        max_attn_len=max_attn_len,
+        contextual_seq_len=contextual_seq_len,
+        min_full_attn_seq_len=min_full_attn_seq_len,
+        q_scale=q_scale,
+        k_scale=k_scale,
+        v_scale=v_scale,
+        tile_config=tile_config,
+    )
+    return out
+
+
+def delta_hstu_mha(
+    max_seq_len: int,
+    alpha: float,
+    delta_q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    seq_offsets: torch.Tensor,
+    num_targets: Optional[torch.Tensor] = None,
+    max_attn_len: int = 0,
+    contextual_seq_len: int = 0,
+    kernel: HammerKernel = HammerKernel.HIP,
+    enable_tma: bool = False,
+    q_scale: float = 1.0,
+    k_scale: float = 1.0,
+    v_scale: float = 1.0,
+    tile_config: int = 0,
+) -> torch.Tensor:
+    """Cached-KV (M-FALCON) forward: ``delta_q`` holds the last ``L // B`` positions of every sequence.
+
+    Returns ``[B * delta_size, H, Dv]`` in the dtype of ``delta_q`` (bf16 for fp8 inputs).
+    """
+    torch._assert(delta_q.dim() == 3, "delta_q must be 3-D")
+    L, H, D = delta_q.shape
+    B = seq_offsets.size(0) - 1
+    torch._assert(B > 0, "seq_offsets must hold at least one sequence")
+    delta_size = L // B
+    torch._assert(max_seq_len > 0, "max_seq_len must be larger than 0")
+    torch._assert(L % B == 0, "delta_q must be padded")
+    torch._assert(k.dim() == 3, "k must be 3-D")
+    torch._assert(k.shape[1] == H, "wrong k shape[1]")
+    torch._assert(k.shape[2] == D, "wrong k shape[2]")
+    torch._assert(v.dim() == 3, "v must be 3-D")
+    torch._assert(v.shape[1] == H, "wrong v shape[1]")
+    torch._assert(v.shape[0] == k.shape[0], "wrong v shape[0]")
+    _require_device(delta_q, "q")
+    _require_device(k, "k")
+    _require_device(v, "v")
+    _require_device(seq_offsets, "seq_offsets")
+    torch._assert(k.dtype == delta_q.dtype and v.dtype == delta_q.dtype, "q, k and v must have the same dtype")
+    if num_targets is not None:
+        _require_device(num_targets, "num_targets")
+        torch._assert(num_targets.numel() == B, "num_targets must have one entry per sequence")
+        num_targets = _index_tensor(num_targets, "num_targets")
+    _check_forward_only(delta_q, k, v)
+    seq_offsets = _index_tensor(seq_offsets, "seq_offsets")
+
+    delta_q = _kernel_layout(delta_q.detach())
+    k = _kernel_layout(k.detach())
+    v = _kernel_layout(v.detach())
+    out_dtype = torch.bfloat16 if delta_q.dtype == torch.float8_e4m3fn else delta_q.dtype
+    out = torch.empty((L, H, v.shape[2]), dtype=out_dtype, device=delta_q.device)
+    if out.numel() == 0:
+        return out
+    hip_backend.mha_fwd(
+        delta_q,
+        k,
+        v,
+        out,
+        seq_offsets,
+        num_targets,
+        max_seq_len=max_seq_len,
+        alpha=alpha,
+        delta_size=delta_size,
+        max_attn_len=max_attn_len,
+        contextual_seq_len=contextual_seq_len,
+        min_full_attn_seq_len=0,
+        q_scale=q_scale,
+        k_scale=k_scale,
+        v_scale=v_scale,
+        tile_config=tile_config,
+    )
+    return out

@@ -1,0 +1,108 @@
+/*
+ * hstu_hip.h -- C ABI of libhstu_hip.so: HSTU jagged attention forward for gfx950 (MI355X).
+ *
+ * This is the boundary a caller binds instead of the reference's native operator
+ * `hstu::hstu_mha_fwd` (generative_recommenders/ops/cpp/hstu_attention/flash_api_cpu.cpp:142-235,
+ * host side flash_common.cpp:394-724).  Plain pointers and sizes only; no torch types.
+ * All pointers are device pointers on the current HIP device.  Calls are asynchronous on the
+ * stream given; nothing is allocated, nothing is read back to the host, no input is modified.
+ *
+ * Semantics (generative_recommenders/ops/pytorch/pt_hstu_attention.py:32-251):
+ *     out[r] = sum_s M(r, s) * silu(alpha * <q_r, k_s>) / max_seq_len * v_s
+ * per sequence b (rows seq_offsets[b] .. seq_offsets[b+1]) and head, where M is the
+ * causal / max_attn_len / contextual_seq_len / num_targets mask of `_get_valid_attn_mask`.
+ */
+#ifndef HSTU_HIP_H_
+#define HSTU_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types of q/k/v.  Output is the same type, except FP8_E4M3 inputs give BF16 output
+ * (flash_common.cpp:596-607). */
+enum HstuDtype { HSTU_BF16 = 0, HSTU_FP16 = 1, HSTU_FP8_E4M3 = 2 };
+
+/* Status codes.  0 is success; the library never throws or aborts. */
+enum HstuStatus {
+    HSTU_OK = 0,
+    HSTU_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+    HSTU_ERR_BAD_DTYPE = -2,      /* dtype not in HstuDtype (flash_common.cpp:428-441) */
+    HSTU_ERR_BAD_HEAD_DIM = -3,   /* head dims this build has no kernel for (flash_common.cpp:591-594) */
+    HSTU_ERR_MISALIGNED = -4,     /* base pointer or a stride breaks 16-byte row alignment (flash_common.cpp:447-452) */
+    HSTU_ERR_BAD_SHAPE = -5,      /* negative / inconsistent sizes, max_seq_len <= 0, delta rows not B*delta */
+    HSTU_ERR_UNSUPPORTED = -6,    /* legal in the reference but not built here */
+    HSTU_ERR_LAUNCH = -7,         /* hipLaunchKernel failed; see hstu_hip_last_error() */
+    HSTU_ERR_BAD_DEVICE = -8      /* the current device is not gfx950 */
+};
+
+/*
+ * Mirrors the subset of `Flash_fwd_params` (ops/cpp/hstu_attention/flash.h:24-110) that the
+ * forward pass uses.  Strides are in ELEMENTS; the innermost (head-dim) stride is 1.
+ */
+typedef struct HstuFwdArgs {
+    const void* q;            /* [total_q,  H, dqk]  (delta mode: [B*delta_size, H, dqk]) */
+    const void* k;            /* [total_kv, H, dqk] */
+    const void* v;            /* [total_kv, H, dv]  */
+    void* out;                /* [total_q,  H, dv]  written for every row of every sequence */
+    int64_t q_row_stride, q_head_stride;
+    int64_t k_row_stride, k_head_stride;
+    int64_t v_row_stride, v_head_stride;
+    int64_t o_row_stride, o_head_stride;
+    const void* seq_offsets;  /* [B+1] monotone, seq_offsets[0] == 0 */
+    const void* num_targets;  /* [B] or NULL */
+    int32_t seq_offsets_i64;  /* 1: int64 elements, 0: int32 (the reference's native op takes int32,
+                                 flash_common.cpp:460-462; its Python callers pass int64) */
+    int32_t num_targets_i64;
+    int32_t batch;            /* B */
+    int32_t heads;            /* H */
+    int32_t dqk;              /* attention dim */
+    int32_t dv;               /* value / output dim */
+    int64_t total_q;          /* rows of q and out */
+    int64_t total_kv;         /* rows of k and v */
+    int32_t max_seq_len;      /* N: upper bound on every sequence length AND the 1/N output scale */
+    int32_t delta_size;       /* 0: q is jagged like k.  >0: q holds the last delta_size positions
+                                 of each sequence (pt_hstu_attention.py:190-251) */
+    float alpha;
+    int32_t max_attn_len;            /* 0 = unlimited */
+    int32_t contextual_seq_len;      /* 0 = none */
+    int32_t min_full_attn_seq_len;   /* 0 = none */
+    int32_t dtype;                   /* HstuDtype */
+    float q_scale, k_scale, v_scale; /* FP8 only: real value = stored value * scale (per tensor) */
+    int32_t tile_config;             /* 0 = choose automatically; otherwise a value of hstu_hip_tile_configs() */
+    int32_t reserved;
+} HstuFwdArgs;
+
+/* Library version, major*10000 + minor*100 + patch. */
+int hstu_hip_version(void);
+
+/* Static, human-readable text for a status code. */
+const char* hstu_hip_status_string(int status);
+
+/* Text of the last HIP runtime error seen by this thread inside the library ("" if none). */
+const char* hstu_hip_last_error(void);
+
+/*
+ * Validate `args` exactly as hstu_hip_mha_fwd would, without touching the device.
+ * Replaces the TORCH_CHECKs of flash_common.cpp:420-594.
+ */
+int hstu_hip_check_args(const HstuFwdArgs* args);
+
+/*
+ * Launch the forward pass on `stream` (a hipStream_t; NULL = the default stream).
+ * Replaces hstu::hstu_mha_fwd (flash_common.cpp:394-724) for both the full and the
+ * delta-query (M-FALCON) forms.
+ */
+int hstu_hip_mha_fwd(const HstuFwdArgs* args, void* stream);
+
+/* Number of selectable tile configurations and a short name for each (1-based ids). */
+int hstu_hip_tile_configs(void);
+const char* hstu_hip_tile_config_name(int id);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_HIP_H_ */

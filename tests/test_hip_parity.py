@@ -1,0 +1,315 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on identical inputs.
+
+bf16 / fp16 tolerance vs the fp32 oracle: max-abs <= 2e-2 and mean-abs <= 2e-3 (the stated bar), plus a
+relative Frobenius bound of 1e-2 because outputs are O(1e-3) and the absolute bounds alone are vacuous.
+"""
+
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_ref, hstu_oracle as O
+
+from util import assert_parity, make_case
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "small_cases.npz")
+
+
+def _announce(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+def _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w=0, c=0, f=0, cfg=0, offs_dtype=torch.int64):
+    out = pkg.hstu_mha(
+        N, alpha, q.to(dev), k.to(dev), v.to(dev), offs.to(offs_dtype).to(dev),
+        num_targets=None if t is None else t.to(offs_dtype).to(dev),
+        max_attn_len=w, contextual_seq_len=c, min_full_attn_seq_len=f, tile_config=cfg,
+    )
+    torch.cuda.synchronize()
+    return out
+
+
+def _ref_full(q, k, v, offs, t, N, alpha, w=0, c=0, f=0, **kw):
+    return O.hstu_mha_per_sequence(
+        N, alpha, q.float(), k.float(), v.float(), offs, num_targets=t, max_attn_len=w, contextual_seq_len=c,
+        min_full_attn_seq_len=f, **kw,
+    )
+
+
+def test_library_is_loaded_from_tree(pkg):
+    from generative_recommenders_amd.ops import hip_backend
+
+    assert hip_backend.lib().hstu_hip_version() >= 100
+    assert os.path.dirname(hip_backend.library_path()).endswith(os.path.join("generative-recommenders_amd", "csrc"))
+
+
+@pytest.mark.parametrize("cfg", [1, 2])
+def test_golden_fixture(pkg, dev, cfg):
+    z = np.load(GOLDEN)
+    for name in sorted({key.split(".")[0] for key in z.files}):
+        _announce("golden", name, "cfg", cfg)
+        q = torch.from_numpy(z[f"{name}.q"]).view(torch.bfloat16)
+        k = torch.from_numpy(z[f"{name}.k"]).view(torch.bfloat16)
+        v = torch.from_numpy(z[f"{name}.v"]).view(torch.bfloat16)
+        offs = torch.from_numpy(z[f"{name}.offsets"])
+        t = torch.from_numpy(z[f"{name}.targets"])
+        t = None if int(t[0]) < 0 else t
+        N, w, c, f, delta = [int(x) for x in z[f"{name}.params"]]
+        alpha = float(z[f"{name}.alpha"][0])
+        want = torch.from_numpy(z[f"{name}.out"])
+        if delta > 0:
+            got = pkg.delta_hstu_mha(
+                N, alpha, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev),
+                max_attn_len=w, contextual_seq_len=c, tile_config=cfg,
+            )
+        else:
+            got = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, c, f, cfg)
+        assert_parity(got, want, name)
+
+
+# the parameter space sampled by ops/tests/hstu_attention_test.py:262-356 of the reference
+REF_GRID = []
+_rng = np.random.default_rng(20240)
+for _i in range(36):
+    REF_GRID.append(
+        dict(
+            seed=100 + _i,
+            B=int(_rng.choice([4, 8])),
+            H=int(_rng.choice([1, 2, 4])),
+            max_uih=int(_rng.choice([20, 100, 128, 256])),
+            max_targets=int(_rng.choice([20, 512])),
+            D=int(_rng.choice([32, 64, 128])),
+            has_targets=bool(_rng.integers(0, 2)),
+            has_window=bool(_rng.integers(0, 2)),
+            c=int(_rng.choice([0, 10])),
+            dtype=[torch.bfloat16, torch.float16][int(_rng.integers(0, 2))],
+            cfg=int(_rng.choice([1, 2])),
+            i32=bool(_rng.integers(0, 2)),
+        )
+    )
+
+
+@pytest.mark.parametrize("p", REF_GRID, ids=[f"g{i}" for i in range(len(REF_GRID))])
+def test_reference_test_grid(pkg, dev, p):
+    _announce("grid", p)
+    rng = np.random.default_rng(p["seed"])
+    B, c = p["B"], p["c"]
+    uih = rng.integers(0, p["max_uih"] + 1, size=B)
+    tg = rng.integers(1, p["max_targets"] + 1, size=B)
+    lengths = uih + tg + c
+    N = p["max_uih"] + p["max_targets"] + c
+    w = int(rng.integers(1, max(2, p["max_uih"] // 5 + 1))) if p["has_window"] else 0
+    q, k, v, offs, t = make_case(p["seed"], lengths, p["H"], p["D"], targets=tg, dtype=p["dtype"])
+    # inputs as the reference test draws them: uniform(-0.1, 0.1)
+    for x in (q, k, v):
+        x.copy_((torch.rand(x.shape, generator=torch.Generator().manual_seed(p["seed"])) * 0.2 - 0.1).to(x.dtype))
+    if not p["has_targets"]:
+        t = None
+    alpha = 1.0 / p["D"] ** 0.5
+    got = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, c, 0, p["cfg"], torch.int32 if p["i32"] else torch.int64)
+    assert_parity(got, _ref_full(q, k, v, offs, t, N, alpha, w, c), str(p))
+
+
+EDGE = [
+    # name, lengths, targets, N, w, c, f
+    ("empty_batch_entries", [0, 5, 0, 0, 130, 0], None, 256, 0, 0, 0),
+    ("all_empty", [0, 0, 0], None, 64, 0, 0, 0),
+    ("single_token", [1, 1, 1], [1, 0, 1], 8, 0, 0, 0),
+    ("tile_multiples", [64, 128, 256, 192, 512], None, 512, 0, 0, 0),
+    ("tile_multiples_pm1", [63, 65, 127, 129, 255, 257], None, 300, 0, 0, 0),
+    ("full_length", [384, 384], None, 384, 0, 0, 0),
+    ("all_targets", [70, 33], [70, 33], 128, 0, 0, 0),
+    ("zero_targets_given", [70, 133], [0, 0], 140, 5, 0, 0),
+    ("window_1", [200, 77], None, 256, 1, 0, 0),
+    ("window_eq_tile", [300, 150], [7, 3], 320, 64, 0, 0),
+    ("window_gt_len", [100, 90], [7, 3], 128, 1000, 3, 0),
+    ("ctx_only_prefix", [40, 300], None, 320, 0, 40, 0),
+    ("ctx_targets_window", [500, 131, 260], [100, 1, 130], 512, 37, 6, 0),
+    ("ctx_big_window_small", [700, 300], [30, 200], 1024, 3, 130, 0),
+    ("min_full", [400, 150, 90], [20, 0, 5], 400, 16, 4, 24),
+    ("min_full_no_targets", [333, 64], None, 400, 10, 0, 50),
+    ("long_one", [2100, 3], [300, 1], 2100, 0, 0, 0),
+    ("long_window_ctx", [1500, 2047], [511, 2], 2048, 256, 6, 0),
+]
+
+
+@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("e", EDGE, ids=[e[0] for e in EDGE])
+def test_edge_cases(pkg, dev, e, cfg):
+    name, lengths, targets, N, w, c, f = e
+    _announce("edge", name, "cfg", cfg)
+    q, k, v, offs, t = make_case(77, lengths, 2, 128, targets=targets)
+    alpha = 1.0 / 128**0.5
+    got = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, c, f, cfg)
+    assert got.shape == v.shape and got.dtype == v.dtype
+    assert_parity(got, _ref_full(q, k, v, offs, t, N, alpha, w, c, f), name)
+
+
+def test_matches_dense_as_written_and_scalar_checker(pkg, dev):
+    """Config 1 of the baseline list (B=8, lengths 16..128, H=2, d=32) in bf16, against all three checkers."""
+    rng = np.random.default_rng(1001)
+    lengths = rng.integers(16, 129, size=8)
+    q, k, v, offs, _ = make_case(1001, lengths, 2, 32)
+    alpha = 1.0 / 32**0.5
+    _announce("cfg1")
+    got = _run_full(pkg, dev, q, k, v, offs, None, 128, alpha)
+    dense = O.pytorch_hstu_mha(128, alpha, q.float(), k.float(), v.float(), offs)
+    assert_parity(got, dense, "dense")
+    assert_parity(got, c_ref.fwd(128, alpha, q, k, v, offs), "scalar C")
+
+
+def test_strided_views_of_one_buffer(pkg, dev):
+    """q, k, v as column slices of one [L, H, 3D] buffer (hstu_compute.py:90-103): same bits as dense copies."""
+    _announce("strided")
+    g = torch.Generator().manual_seed(5)
+    lengths = torch.tensor([300, 90, 200])
+    offs = torch.zeros(4, dtype=torch.int64)
+    offs[1:] = torch.cumsum(lengths, 0)
+    L, H, D = int(offs[-1]), 4, 128
+    x = (torch.randn((L, H, 3 * D), generator=g) * 0.1).to(torch.bfloat16).to(dev)
+    q, k, v = torch.split(x, [D, D, D], dim=-1)
+    assert not q.is_contiguous()
+    a = pkg.hstu_mha(320, 0.1, q, k, v, offs.to(dev))
+    b = pkg.hstu_mha(320, 0.1, q.contiguous(), k.contiguous(), v.contiguous(), offs.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert_parity(a, _ref_full(q.cpu(), k.cpu(), v.cpu(), offs, None, 320, 0.1), "strided")
+
+
+def test_inputs_not_modified_and_rows_all_written(pkg, dev):
+    _announce("inputs untouched")
+    q, k, v, offs, t = make_case(9, [100, 0, 257], 2, 64, targets=[3, 0, 100])
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = pkg.hstu_mha(300, 0.2, qd, kd, vd, offs.to(dev), num_targets=t.to(dev), max_attn_len=20)
+    torch.cuda.synchronize()
+    assert torch.equal(qd.cpu(), q) and torch.equal(kd.cpu(), k) and torch.equal(vd.cpu(), v)
+    assert torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("delta,w,c,D", [(8, 0, 0, 128), (256, 0, 0, 128), (130, 50, 4, 64), (1, 0, 0, 32), (20, 7, 0, 128)])
+def test_delta_against_oracle_and_tail_of_full(pkg, dev, delta, w, c, D, cfg):
+    """delta_hstu_mha vs the oracle, and == the last rows of hstu_mha (hstu_attention_test.py:382-488)."""
+    _announce("delta", delta, w, c, D, cfg)
+    rng = np.random.default_rng(delta)
+    lengths = rng.integers(0, 400, size=5) + delta + c
+    q, k, v, offs, t = make_case(31 + delta, lengths, 2, D, targets=[delta] * 5)
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(5)])
+    dq = q[idx].contiguous()
+    N = int(lengths.max()) + 3
+    alpha = 1.0 / D**0.5
+    got = pkg.delta_hstu_mha(
+        N, alpha, dq.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev), max_attn_len=w,
+        contextual_seq_len=c, tile_config=cfg,
+    )
+    torch.cuda.synchronize()
+    assert got.shape == (5 * delta, 2, D)
+    ref = O.cached_hstu_mha_per_sequence(N, alpha, dq.float(), k.float(), v.float(), offs, t, w, c)
+    assert_parity(got, ref, "delta vs oracle")
+    full = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, c, 0, cfg)
+    assert_parity(got, full[idx.to(dev)], "delta vs tail of full", rel_tol=2e-3)
+
+
+def test_invariants_on_device(pkg, dev):
+    """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
+    permuting two targets permutes the outputs (stu_test.py:180-321)."""
+    _announce("invariants")
+    lengths = [700, 130, 512]
+    q, k, v, offs, t = make_case(13, lengths, 4, 128, targets=[50, 3, 0])
+    kw = dict(w=100, c=5)
+    a = _run_full(pkg, dev, q, k, v, offs, t, 1024, 0.09, **kw)
+    b = _run_full(pkg, dev, q, k, v, offs, t, 2048, 0.09, **kw)
+    assert torch.equal(a.float(), b.float() * 2.0)
+    s0, s1 = int(offs[1]), int(offs[2])
+    alone = _run_full(pkg, dev, q[s0:s1], k[s0:s1], v[s0:s1], torch.tensor([0, s1 - s0]), t[1:2], 1024, 0.09, **kw)
+    assert torch.equal(alone, a[s0:s1])
+    h2 = _run_full(pkg, dev, q[:, 2:3].contiguous(), k[:, 2:3].contiguous(), v[:, 2:3].contiguous(), offs, t, 1024, 0.09, **kw)
+    assert torch.equal(h2, a[:, 2:3])
+    perm = torch.arange(q.shape[0])
+    perm[699], perm[660] = 660, 699
+    c = _run_full(pkg, dev, q[perm], k[perm], v[perm], offs, t, 1024, 0.09, **kw)
+    assert torch.equal(c, a[perm.to(dev)])
+
+
+def test_cfg2_shape_subset(pkg, dev):
+    """Baseline config 2 (B=256, lengths 64..1024, H=4, d=128) at full size; oracle on a subset of sequences."""
+    from generative_recommenders_amd import workloads
+
+    wl = workloads.make_workload("cfg2")
+    inp = workloads.make_inputs(wl, torch.device("cpu"))
+    _announce("cfg2 full size", wl.total_kv)
+    got = _run_full(pkg, dev, inp["q"], inp["k"], inp["v"], inp["seq_offsets"], None, wl.max_seq_len, wl.alpha)
+    seqs = [0, 1, 17, 100, 255, int(np.argmax(wl.lengths)), int(np.argmin(wl.lengths))]
+    ref = _ref_full(inp["q"], inp["k"], inp["v"], inp["seq_offsets"], None, wl.max_seq_len, wl.alpha, sequences=seqs)
+    offs = inp["seq_offsets"]
+    for b in seqs:
+        s0, s1 = int(offs[b]), int(offs[b + 1])
+        assert_parity(got[s0:s1], ref[s0:s1], f"cfg2 seq {b}")
+
+
+def test_cfg3_shape_subset(pkg, dev):
+    """Baseline config 3 (Zipf lengths to 8192, window 2048, 6 contextual, targets) at full size."""
+    from generative_recommenders_amd import workloads
+
+    wl = workloads.make_workload("cfg3")
+    inp = workloads.make_inputs(wl, torch.device("cpu"))
+    _announce("cfg3 full size", wl.total_kv)
+    got = _run_full(
+        pkg, dev, inp["q"], inp["k"], inp["v"], inp["seq_offsets"], inp["num_targets"], wl.max_seq_len, wl.alpha,
+        wl.max_attn_len, wl.contextual_seq_len,
+    )
+    order = np.argsort(wl.lengths)
+    seqs = [int(order[-1]), int(order[0]), int(order[len(order) // 2]), 0]
+    mids = [int(b) for b in range(wl.batch) if 256 < wl.lengths[b] < 8192][:2]
+    seqs = sorted(set(seqs + mids))
+    ref = _ref_full(
+        inp["q"], inp["k"], inp["v"], inp["seq_offsets"], inp["num_targets"], wl.max_seq_len, wl.alpha,
+        wl.max_attn_len, wl.contextual_seq_len, sequences=seqs,
+    )
+    offs = inp["seq_offsets"]
+    for b in seqs:
+        s0, s1 = int(offs[b]), int(offs[b + 1])
+        assert_parity(got[s0:s1], ref[s0:s1], f"cfg3 seq {b} n={s1 - s0}")
+
+
+def test_cfg4_shape_subset(pkg, dev):
+    """Baseline config 4 (M-FALCON: 32 users, history 1024..4096, 256 delta queries) at full size."""
+    from generative_recommenders_amd import workloads
+
+    wl = workloads.make_workload("cfg4")
+    inp = workloads.make_inputs(wl, torch.device("cpu"))
+    _announce("cfg4 full size", wl.total_kv)
+    got = pkg.delta_hstu_mha(
+        wl.max_seq_len, wl.alpha, inp["q"].to(dev), inp["k"].to(dev), inp["v"].to(dev), inp["seq_offsets"].to(dev),
+        num_targets=inp["num_targets"].to(dev),
+    )
+    torch.cuda.synchronize()
+    seqs = [0, 7, 31, int(np.argmax(wl.lengths))]
+    ref = O.cached_hstu_mha_per_sequence(
+        wl.max_seq_len, wl.alpha, inp["q"].float(), inp["k"].float(), inp["v"].float(), inp["seq_offsets"],
+        inp["num_targets"], sequences=seqs,
+    )
+    for b in seqs:
+        assert_parity(got[b * 256 : (b + 1) * 256], ref[b * 256 : (b + 1) * 256], f"cfg4 user {b}")
+
+
+def test_wrapper_rejects_what_it_cannot_do(pkg, dev):
+    q, k, v, offs, _ = make_case(1, [10, 20], 2, 32)
+    with pytest.raises(AssertionError):
+        pkg.hstu_mha(0, 0.1, q.to(dev), k.to(dev), v.to(dev), offs.to(dev))
+    with pytest.raises(AssertionError):
+        pkg.hstu_mha(32, 0.1, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), causal=False)
+    with pytest.raises(RuntimeError):
+        pkg.hstu_mha(32, 0.1, q.float().to(dev), k.float().to(dev), v.float().to(dev), offs.to(dev))
+    qg = q.to(dev).requires_grad_()
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_mha(32, 0.1, qg, k.to(dev), v.to(dev), offs.to(dev))
+    with torch.no_grad():
+        pkg.hstu_mha(32, 0.1, qg, k.to(dev), v.to(dev), offs.to(dev))
+    torch.cuda.synchronize()

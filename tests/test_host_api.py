@@ -1,0 +1,166 @@
+"""CPU tests of the host side: the C-ABI library loads and exports what include/hstu_hip.h declares,
+argument validation returns the documented status codes, the Python mirror keeps the reference's
+assertions, and the work counts used by the benchmark are exact.  No kernel is launched."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_ref
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def backend():
+    from generative_recommenders_amd.ops import hip_backend
+
+    if not os.path.exists(hip_backend.library_path()):
+        import __graft_entry__
+
+        __graft_entry__.build()
+    return hip_backend
+
+
+def test_library_exports_every_declared_symbol(backend):
+    header = open(os.path.join(ROOT, "include", "hstu_hip.h")).read()
+    declared = set(re.findall(r"\b(hstu_hip_\w+)\s*\(", header))
+    assert declared == set(backend.EXPORTS), declared ^ set(backend.EXPORTS)
+    lib = ctypes.CDLL(backend.library_path())
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert backend.lib().hstu_hip_version() >= 100
+    assert backend.tile_config_names()[0] == "m128n64w4"
+
+
+def test_struct_mirror_has_the_header_fields_in_order(backend):
+    header = open(os.path.join(ROOT, "include", "hstu_hip.h")).read()
+    body = header[header.index("typedef struct HstuFwdArgs {") : header.index("} HstuFwdArgs;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S).replace("typedef struct HstuFwdArgs {", "")
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        parts = decl.split(",")
+        names.append(re.findall(r"(\w+)\s*$", parts[0].strip())[0])
+        names += [p.strip() for p in parts[1:]]
+    assert names == [f[0] for f in backend.HstuFwdArgs._fields_]
+
+
+def _args(backend, **over):
+    a = backend.HstuFwdArgs()
+    a.q = a.k = a.v = a.out = 0x1000
+    a.seq_offsets = 0x2000
+    for s in ("q", "k", "v", "o"):
+        setattr(a, f"{s}_row_stride", 4 * 128)
+        setattr(a, f"{s}_head_stride", 128)
+    a.batch, a.heads, a.dqk, a.dv = 2, 4, 128, 128
+    a.total_q = a.total_kv = 100
+    a.max_seq_len = 64
+    a.alpha = 0.1
+    a.seq_offsets_i64 = 1
+    for key, val in over.items():
+        setattr(a, key, val)
+    return a
+
+
+def test_check_args_status_codes(backend):
+    chk = lambda **o: backend.lib().hstu_hip_check_args(ctypes.byref(_args(backend, **o)))  # noqa: E731
+    assert chk() == 0
+    assert backend.lib().hstu_hip_check_args(None) == -1
+    assert chk(q=None) == -1
+    assert chk(seq_offsets=None) == -1
+    assert chk(dtype=7) == -2
+    assert chk(dqk=48, dv=48) == -3
+    assert chk(dqk=64, dv=128) == -3
+    assert chk(q=0x1008) == -4
+    assert chk(k_row_stride=4 * 128 + 4) == -4
+    assert chk(max_seq_len=0) == -5
+    assert chk(total_q=99) == -5
+    assert chk(delta_size=8, total_q=17) == -5
+    assert chk(delta_size=8, total_q=16) == 0
+    assert chk(tile_config=99) == -5
+    assert chk(total_q=0, total_kv=0, q=None) == 0  # empty input: nothing is dereferenced
+    for rc in range(-8, 1):
+        assert backend.lib().hstu_hip_status_string(rc)
+    with pytest.raises(RuntimeError):
+        backend.raise_for_status(-3)
+    with pytest.raises(ValueError):
+        backend.raise_for_status(-5)
+
+
+def test_python_mirror_keeps_reference_assertions(pkg):
+    q = torch.zeros(10, 2, 32, dtype=torch.bfloat16)
+    offs = torch.tensor([0, 10])
+    with pytest.raises(AssertionError, match="max_seq_len must be larger than 0"):
+        pkg.hstu_mha(0, 0.1, q, q, q, offs)
+    with pytest.raises(AssertionError, match="q must be 3-D"):
+        pkg.hstu_mha(16, 0.1, q[0], q[0], q, offs)
+    with pytest.raises(AssertionError, match="k must be the same shape as q"):
+        pkg.hstu_mha(16, 0.1, q, q[:5], q, offs)
+    with pytest.raises(AssertionError, match="only support causal attention"):
+        pkg.hstu_mha(16, 0.1, q, q, q, offs, causal=False)
+    # CPU tensors are refused: there is no fallback path
+    with pytest.raises(AssertionError, match="q must be CUDA tensor"):
+        pkg.hstu_mha(16, 0.1, q, q, q, offs)
+    with pytest.raises(AssertionError, match="delta_q must be padded"):
+        pkg.delta_hstu_mha(16, 0.1, q[:9], q, q, torch.tensor([0, 4, 10]))
+    with pytest.raises(AssertionError, match="wrong k shape"):
+        pkg.delta_hstu_mha(16, 0.1, q[:8], q[:, :1], q, torch.tensor([0, 4, 10]))
+
+
+def test_package_does_not_import_the_oracle():
+    pkg_dir = os.path.join(ROOT, "generative-recommenders_amd")
+    for dirpath, _, files in os.walk(pkg_dir):
+        for fn in files:
+            if fn.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, fn)).read()
+                assert "oracle" not in text, os.path.join(dirpath, fn)
+
+
+def test_valid_pair_counts_match_brute_force():
+    from generative_recommenders_amd import workloads
+
+    rng = np.random.default_rng(3)
+    checked = 0
+    for _ in range(400):
+        n = int(rng.integers(1, 80))
+        c = int(rng.choice([0, 0, 1, 6]))
+        t = int(rng.integers(0, max(1, n - c) + 1)) if rng.random() < 0.7 else 0
+        if n - t < c:
+            continue
+        w = int(rng.choice([0, 1, 7, 30, 200]))
+        f = int(rng.choice([0, 0, 3]))
+        rows = workloads.valid_pairs_per_row(n, t, w, c, f)
+        m = c_ref.mask(n, c, t, w, f)
+        assert (rows == m.sum(1)).all(), (n, c, t, w, f)
+        d = int(rng.integers(1, n + 1))
+        assert rows[n - d :].sum() == c_ref.count_pairs(n, c, t, w, f, d)
+        checked += 1
+    assert checked > 300
+
+
+def test_workload_definitions():
+    from generative_recommenders_amd import workloads
+
+    h = workloads.make_workload("headline")
+    assert (h.batch, h.heads, h.dqk, h.max_seq_len) == (64, 4, 128, 8192)
+    pairs = workloads.count_valid_pairs(h)
+    assert pairs == 64 * (8192 * 8193 // 2)
+    assert workloads.algorithmic_flops(h) == 2 * 256 * 4 * pairs
+    # the reference bench's n^2/2 convention agrees with the exact count to 1/n for plain causal
+    assert abs(workloads.reference_convention_flops(h) / workloads.algorithmic_flops(h) - 1) < 2e-4
+    c3 = workloads.make_workload("cfg3")
+    assert c3.lengths.min() >= 256 and c3.lengths.max() <= 8192
+    assert (c3.num_targets >= 1).all() and (c3.lengths - c3.num_targets >= 7).all()
+    c4 = workloads.make_workload("cfg4")
+    assert c4.total_q == 32 * 256 and c4.max_seq_len == 4352
+    for name in workloads.WORKLOADS:
+        wl = workloads.make_workload(name)
+        assert wl.lengths.max() <= wl.max_seq_len
+        assert workloads.algorithmic_bytes(wl) > 0
