@@ -109,6 +109,9 @@ def test_reference_test_grid(pkg, dev, p):
     # inputs as the reference test draws them: uniform(-0.1, 0.1)
     for x in (q, k, v):
         x.copy_((torch.rand(x.shape, generator=torch.Generator().manual_seed(p["seed"])) * 0.2 - 0.1).to(x.dtype))
+    if p["dtype"] == torch.float16:
+        # outputs of O(1e-6) would be fp16 subnormals (quantum 6e-8); the op is linear in v, so lift v instead
+        v.mul_(1024.0)
     if not p["has_targets"]:
         t = None
     alpha = 1.0 / p["D"] ** 0.5
