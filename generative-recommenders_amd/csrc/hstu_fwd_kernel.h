@@ -103,14 +103,43 @@ struct SeqMask {
     }
 };
 
+// Chunk swizzles.  LDS has 64 banks of 4 bytes (256 bytes per clock); a row of CH 16-byte chunks is
+// stored with chunk index XOR f(row).
+//
+// K tile, read with ds_read_b128 by 16 lanes at a time (16 consecutive rows, same logical chunk): f must
+// send those 16 rows to 16 different 16-byte slots of the 256-byte bank line.
 template <int CH>
-__device__ __forceinline__ int swz(int row) {
-    return row & ((CH < 16 ? CH : 16) - 1);
+__device__ __forceinline__ int swz_k(int row) {
+    static_assert(CH == 4 || CH == 8 || CH == 16, "row of 64, 128 or 256 bytes");
+    return (row / (16 / CH)) & (CH - 1);
+}
+// V tile, read with ds_read_b64_tr_b16: one instruction touches 8 rows (4 per half-wave) x one 64-byte
+// segment, 8 bytes per lane.  f must send rows r..r+3 to four different 64-byte bank groups and rows
+// r, r+4 to different 32-byte halves of a group.
+template <int CH>
+__device__ __forceinline__ int swz_v(int row) {
+    static_assert(CH == 4 || CH == 8 || CH == 16, "row of 64, 128 or 256 bytes");
+    const int half_swap = ((row >> 2) & 1) << 1;
+    if (CH == 16) return ((row & 3) << 2) | half_swap;
+    if (CH == 8) return (((row >> 1) & 1) << 2) | half_swap;
+    return half_swap;
+}
+
+// 16 bytes per lane, global memory -> LDS at lds_base + 16*lane (lds_base is wave-uniform and goes
+// through M0).  Written as inline assembly on purpose: the compiler then does not know that an LDS
+// write is in flight and does not put a vmcnt(0) wait in front of the next LDS read, which would
+// expose the whole HBM latency of the prefetch.  The kernel waits for these copies itself
+// (s_waitcnt vmcnt(0) followed by the workgroup barrier) before the tile is read.  The s_nop covers the
+// one wait state the hardware wants between a scalar write of M0 and an LDS-DMA instruction; the
+// compiler's hazard pass does not look inside an asm block.
+__device__ __forceinline__ void global_load_lds16(const char* src, const char* lds_base) {
+    const unsigned m0 = (unsigned)(uintptr_t)HSTU_LDS(const char, lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0), "v"(src) : "memory");
 }
 
 // Copy `ROWS` rows of `ROWBYTES` bytes from global memory into LDS with the chunk swizzle.
 // Rows at or beyond `n_rows_valid` re-read the last valid row (their products are masked).
-template <int ROWS, int ROWBYTES, int NTHREADS>
+template <int ROWS, int ROWBYTES, int NTHREADS, bool IS_V>
 __device__ __forceinline__ void load_tile_to_lds(const char* gbase, int64_t row_stride_bytes, int row0,
                                                  int last_row, char* lds_tile, int wave, int lane) {
     constexpr int CH = ROWBYTES / 16;                // 16-byte chunks per row
@@ -123,11 +152,11 @@ __device__ __forceinline__ void load_tile_to_lds(const char* gbase, int64_t row_
         int p = inst * 64 + lane;
         int row = p / CH;
         int phys = p % CH;
-        int logical = phys ^ swz<CH>(row);
+        int logical = phys ^ (IS_V ? swz_v<CH>(row) : swz_k<CH>(row));
         int grow = row0 + row;
         grow = grow > last_row ? last_row : grow;
         const char* src = gbase + (int64_t)grow * row_stride_bytes + logical * 16;
-        __builtin_amdgcn_global_load_lds(HSTU_GLB(void, src), HSTU_LDS(void, lds_tile + inst * 1024), 16, 0, 0);
+        global_load_lds16(src, lds_tile + inst * 1024);
     }
 }
 
@@ -276,8 +305,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     const int64_t k_rsb = p.k_rs * 2, v_rsb = p.v_rs * 2;
 
     if (jt < jt_end) {
-        load_tile_to_lds<BN, KROW, NT>(kbase, k_rsb, jt * BN, n - 1, smem, wave, lane);
-        load_tile_to_lds<BN, VROW, NT>(vbase, v_rsb, jt * BN, n - 1, smem + KTILE, wave, lane);
+        load_tile_to_lds<BN, KROW, NT, false>(kbase, k_rsb, jt * BN, n - 1, smem, wave, lane);
+        load_tile_to_lds<BN, VROW, NT, true>(vbase, v_rsb, jt * BN, n - 1, smem + KTILE, wave, lane);
     }
 
     // ---- Q operand (B of the first product): lane holds Q[row l32][16 ks + 8 g .. +8)
@@ -312,7 +341,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     // K, A operand: row sub*32 + l32, logical chunk 2 ks + g
     int kaddr[KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = l32 * KROW + (((2 * ks + g) ^ swz<KCH>(l32)) * 16);
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = l32 * KROW + (((2 * ks + g) ^ swz_k<KCH>(l32)) * 16);
     // V^T, A operand via ds_read_b64_tr_b16.  Within each group of 16 lanes, lane 4j+q supplies the
     // address of 4 consecutive dv of kv row j; the hardware hands lane i the four kv rows of dv i.
     // Operand lane l must end up with dv = l32 and kv slots {4g+0..3} (first read), {8+4g+0..3} (second).
@@ -326,7 +355,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 int chunk = dt * 4 + 2 * half + (q4 >> 1);
-                vaddr[sec][dt] = row * VROW + ((chunk ^ swz<VCH>(row)) * 16) + (q4 & 1) * 8;
+                vaddr[sec][dt] = row * VROW + ((chunk ^ swz_v<VCH>(row)) * 16) + (q4 & 1) * 8;
             }
         }
     }
@@ -348,8 +377,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
         __syncthreads();                      // ... for every wave, and the other stage is no longer read
         if (jn < jt_end) {
             char* nxt = smem + (stage ^ 1) * STAGE;
-            load_tile_to_lds<BN, KROW, NT>(kbase, k_rsb, jn * BN, n - 1, nxt, wave, lane);
-            load_tile_to_lds<BN, VROW, NT>(vbase, v_rsb, jn * BN, n - 1, nxt + KTILE, wave, lane);
+            load_tile_to_lds<BN, KROW, NT, false>(kbase, k_rsb, jn * BN, n - 1, nxt, wave, lane);
+            load_tile_to_lds<BN, VROW, NT, true>(vbase, v_rsb, jn * BN, n - 1, nxt + KTILE, wave, lane);
         }
 
         const int cls = M.classify(wR0, wR1, jt * BN, BN);
