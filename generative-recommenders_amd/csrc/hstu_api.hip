@@ -8,6 +8,7 @@
 #include <cstring>
 
 #include "hstu_fwd_kernel.h"
+#include "hstu_fwd_pp_kernel.h"
 
 namespace {
 
@@ -24,7 +25,7 @@ struct TileConfig {
 // id 1..: see hstu_hip_tile_configs()
 const TileConfig kConfigs[] = {
     {"m128n64w4", 1, 4, 64},
-    {"m256n64w4", 2, 4, 64},
+    {"m256n64w8pp", 1, 8, 64},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -56,12 +57,29 @@ int launch(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
     return HSTU_OK;
 }
 
+template <class TT, int DQK, int DV, int BN>
+int launch_pp(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
+    constexpr int smem = 0;  // the kernel's LDS is a static array
+    auto kern = hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN>;
+    const int pairs_per_xcd = (num_pairs + 7) / 8;
+    const long long grid = (long long)pairs_per_xcd * 8 * p.num_mb;
+    if (grid <= 0) return HSTU_OK;
+    if (grid > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_last_error("kernel launch", e);
+        return HSTU_ERR_LAUNCH;
+    }
+    return HSTU_OK;
+}
+
 template <class TT, int D>
 int launch_cfg(const hstu::FwdParams& p0, int cfg, int rows_per_pair, int num_pairs, hipStream_t stream) {
     hstu::FwdParams p = p0;
     if (cfg == 2) {
         p.num_mb = (rows_per_pair + 255) / 256;
-        return launch<TT, D, D, 2, 4, 64, 1>(p, num_pairs, stream);
+        return launch_pp<TT, D, D, 64>(p, num_pairs, stream);
     }
     p.num_mb = (rows_per_pair + 127) / 128;
     return launch<TT, D, D, 1, 4, 64, 2>(p, num_pairs, stream);

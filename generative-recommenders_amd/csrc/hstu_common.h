@@ -1,0 +1,374 @@
+// HSTU jagged attention forward for gfx950 (CDNA4): device code.
+//
+// One workgroup owns BM = NW*QT*32 consecutive query rows of one (sequence, head) pair and walks
+// the key/value rows of that sequence in tiles of BN.  All matrix work is on
+// v_mfma_f32_32x32x16_{bf16,f16}, computed transposed so that no register shuffle is needed
+// between the two products:
+//
+//   S^T[kv, q] = K[kv, :] . Q[q, :]^T        A = K tile (LDS),   B = Q (registers, loaded once)
+//   P^T        = silu-part(S^T), masked      in registers, packed to 16 bit
+//   O^T[dv, q] += V^T[dv, kv] . P^T[kv, q]   A = V tile (LDS, transposing read), B = P^T (registers)
+//
+// The accumulator layout of a 32x32 MFMA holds, per lane, one column (a query row) and sixteen
+// rows (kv positions); taken eight at a time those sixteen values are exactly the B operand of
+// the second product, provided the A operand (V^T) enumerates the kv rows in the same order,
+// which the ds_read_b64_tr_b16 addressing below arranges.
+//
+// silu(alpha*s)/N is evaluated as  s * rcp(1 + exp2(-alpha*log2(e)*s))  per element and the
+// common factor alpha/N is applied once to the fp32 output.  There is no row max / row sum:
+// HSTU attention is pointwise (pt_hstu_attention.py:151-182 of the reference).
+//
+// K and V tiles go HBM -> LDS with global_load_lds_dwordx4 (no register staging), double
+// buffered.  An XOR swizzle of the 16-byte chunk index with the row index keeps both the
+// b128 reads of K and the transposing reads of V off each other's banks; it is applied on the
+// global side of the copy because the LDS side of a direct load is fixed (lane i -> base + 16 i).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hstu {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+
+#define HSTU_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define HSTU_GLB(T, p) ((const __attribute__((address_space(1))) T*)(p))
+
+__device__ __forceinline__ int64_t uniform64(int64_t x) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(uint64_t)x);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)((uint64_t)x >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+struct FwdParams {
+    const char* q;
+    const char* k;
+    const char* v;
+    char* o;
+    int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;  // strides in elements
+    const void* offsets;
+    const void* targets;
+    int offsets_i64, targets_i64;
+    int B, H;
+    int num_mb;         // row blocks per (sequence, head) pair in the grid
+    int max_seq_len;
+    int delta;          // 0 = full attention
+    int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
+    float c1;           // -alpha * log2(e)
+    float oscale;       // alpha / max_seq_len
+};
+
+struct Bf16 {
+    typedef bf16x8_t vec8;
+    typedef __bf16 elem;
+    static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+struct Fp16 {
+    typedef f16x8_t vec8;
+    typedef _Float16 elem;
+    static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+// Per-sequence mask state; every field is wave-uniform.
+struct SeqMask {
+    int n;        // sequence length
+    int shift;    // contextual_seq_len - 1 (0 if none): position -> id is max(pos - shift, 0)
+    int idclamp;  // ids are clamped to this (max_id when targets are given, else INT_MAX)
+    int max_id;   // id of the first target (or one past the last id)
+    int w, c, f;
+    __device__ __forceinline__ int id(int pos) const {
+        int x = pos - shift;
+        x = x < 0 ? 0 : x;
+        return x > idclamp ? idclamp : x;
+    }
+    // Classify rows [r_lo, r_hi] (inclusive, all < n) against kv positions [s_lo, s_lo + bn):
+    // 0 = no valid pair, 1 = some, 2 = every pair valid and no padding column.
+    __device__ __forceinline__ int classify(int r_lo, int r_hi, int s_lo, int bn) const {
+        if (s_lo >= n || r_hi < r_lo) return 0;
+        int s_hi = s_lo + bn - 1;
+        bool padded = s_hi >= n;
+        if (padded) s_hi = n - 1;
+        int idr_lo = id(r_lo), idr_hi = id(r_hi), ids_lo = id(s_lo), ids_hi = id(s_hi);
+        if (!padded && ids_hi < idr_lo && (w == 0 || idr_hi - ids_lo <= w)) return 2;
+        bool diag = s_lo <= r_hi && r_lo <= s_hi;
+        bool caus = ids_lo < idr_hi && (w == 0 || f > 0 || idr_lo - ids_hi <= w);
+        bool ctx = c > 0 && idr_lo == 0 && ids_lo < max_id;
+        return (diag || caus || ctx) ? 1 : 0;
+    }
+};
+
+// Chunk swizzles.  LDS has 64 banks of 4 bytes (256 bytes per clock); a row of CH 16-byte chunks is
+// stored with chunk index XOR f(row).
+//
+// K tile, read with ds_read_b128 by 16 lanes at a time (16 consecutive rows, same logical chunk): f must
+// send those 16 rows to 16 different 16-byte slots of the 256-byte bank line.
+template <int CH>
+__device__ __forceinline__ int swz_k(int row) {
+    static_assert(CH == 4 || CH == 8 || CH == 16, "row of 64, 128 or 256 bytes");
+    return (row / (16 / CH)) & (CH - 1);
+}
+// V tile, read with ds_read_b64_tr_b16: one instruction touches 8 rows (4 per half-wave) x one 64-byte
+// segment, 8 bytes per lane.  f must send rows r..r+3 to four different 64-byte bank groups and rows
+// r, r+4 to different 32-byte halves of a group.
+template <int CH>
+__device__ __forceinline__ int swz_v(int row) {
+    static_assert(CH == 4 || CH == 8 || CH == 16, "row of 64, 128 or 256 bytes");
+    const int half_swap = ((row >> 2) & 1) << 1;
+    if (CH == 16) return ((row & 3) << 2) | half_swap;
+    if (CH == 8) return (((row >> 1) & 1) << 2) | half_swap;
+    return half_swap;
+}
+
+// 16 bytes per lane, global memory -> LDS at lds_base + 16*lane (lds_base is wave-uniform and goes
+// through M0).  Written as inline assembly on purpose: the compiler then does not know that an LDS
+// write is in flight and does not put a vmcnt(0) wait in front of the next LDS read, which would
+// expose the whole HBM latency of the prefetch.  The kernel waits for these copies itself
+// (s_waitcnt vmcnt(0) followed by the workgroup barrier) before the tile is read.  The s_nop covers the
+// one wait state the hardware wants between a scalar write of M0 and an LDS-DMA instruction; the
+// compiler's hazard pass does not look inside an asm block.
+__device__ __forceinline__ void global_load_lds16(const char* src, const char* lds_base) {
+    const unsigned m0 = (unsigned)(uintptr_t)HSTU_LDS(const char, lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0), "v"(src) : "memory");
+}
+
+// What one workgroup has to do; every field is wave-uniform.
+struct Work {
+    int b, h;
+    int64_t seq_start;
+    int n;            // sequence length (clipped to max_seq_len)
+    int nq;           // query rows of this sequence (n, or delta_size)
+    int m0;           // first query row of the workgroup (index into the nq rows)
+    int rbase;        // sequence position of query row 0 (n - delta_size in delta mode)
+    int u;            // number of non-target positions
+    int R0, R1;       // sequence positions of the workgroup's first and last row (inclusive)
+    int jt_begin;     // first kv tile that can hold a valid pair
+    int jt_end;       // one past the last such tile
+    bool skip_scan;   // true if tiles inside [jt_begin, jt_end) may hold no valid pair (window / targets / contextual)
+    SeqMask M;
+};
+
+// Decode blockIdx.x.  Workgroup ids go round-robin over the 8 XCDs, so ids congruent mod 8 share
+// an L2: all row blocks of one (sequence, head) pair stay on one XCD, heaviest (last) block first.
+// Returns false if this workgroup has nothing to do.
+template <int BM, int BN>
+__device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
+    const int bid = blockIdx.x;
+    const int xcd = bid & 7;
+    const int slot = bid >> 3;
+    const int pair = (slot / p.num_mb) * 8 + xcd;
+    if (pair >= p.B * p.H) return false;
+    const int mb = p.num_mb - 1 - (slot % p.num_mb);
+    w.b = pair / p.H;
+    w.h = pair - w.b * p.H;
+    int64_t seq_start, seq_end;
+    if (p.offsets_i64) {
+        seq_start = ((const int64_t*)p.offsets)[w.b];
+        seq_end = ((const int64_t*)p.offsets)[w.b + 1];
+    } else {
+        seq_start = ((const int*)p.offsets)[w.b];
+        seq_end = ((const int*)p.offsets)[w.b + 1];
+    }
+    // Values read from memory are the same for every lane; say so, so that everything derived from
+    // them (loop bounds, tile classes, base addresses) lives in scalar registers.
+    w.seq_start = uniform64(seq_start);
+    int n = __builtin_amdgcn_readfirstlane((int)(seq_end - seq_start));
+    n = n > p.max_seq_len ? p.max_seq_len : n;  // rows past max_seq_len do not exist for the reference either
+    w.n = n;
+    w.nq = p.delta > 0 ? p.delta : n;
+    w.m0 = mb * BM;
+    w.rbase = p.delta > 0 ? n - p.delta : 0;
+    if (n <= 0 || w.m0 >= w.nq || w.rbase < 0) return false;
+
+    int t = 0;
+    if (p.targets) t = p.targets_i64 ? (int)((const int64_t*)p.targets)[w.b] : ((const int*)p.targets)[w.b];
+    t = __builtin_amdgcn_readfirstlane(t);
+    SeqMask& M = w.M;
+    M.n = n;
+    M.w = p.w;
+    M.c = p.c;
+    M.f = p.f;
+    M.shift = p.c > 0 ? p.c - 1 : 0;
+    w.u = n - t;
+    M.max_id = w.u - M.shift;
+    M.idclamp = p.targets ? M.max_id : 0x7fffffff;
+
+    const int m1 = (w.m0 + BM < w.nq ? w.m0 + BM : w.nq);
+    w.R0 = w.rbase + w.m0;
+    w.R1 = w.rbase + m1 - 1;
+    const int idr_lo = M.id(w.R0);
+    const bool ctx_rows = p.c > 0 && idr_lo == 0;
+    int kv_hi = w.R1 + 1;
+    if (ctx_rows && w.u > kv_hi) kv_hi = w.u;
+    if (kv_hi > n) kv_hi = n;
+    int kv_lo = 0;
+    if (p.w > 0 && p.f == 0 && !ctx_rows && idr_lo - p.w > 0) kv_lo = idr_lo - p.w + M.shift;
+    w.jt_end = (kv_hi + BN - 1) / BN;
+    w.jt_begin = kv_lo / BN;
+    w.skip_scan = p.w > 0 || p.c > 0 || p.targets != nullptr;
+    return true;
+}
+
+// First tile index >= jt that holds a valid pair for the workgroup's rows (jt_end if none).
+template <int BN>
+__device__ __forceinline__ int next_valid_tile(const Work& w, int jt) {
+    if (w.skip_scan)
+        while (jt < w.jt_end && w.M.classify(w.R0, w.R1, jt * BN, BN) == 0) ++jt;
+    return jt;
+}
+
+// Per-lane constants of the mask predicate for one query row.
+struct RowMask {
+    int pos;    // sequence position of the row
+    int lo;     // id(row) - window: key ids in [lo, lo + w) pass the causal+window test
+    int w;      // window of this row (INT_MAX if unlimited)
+    bool ctx;   // contextual row: sees every non-target key
+    __device__ __forceinline__ void init(const SeqMask& M, int row_pos) {
+        const int idr = M.id(row_pos);
+        pos = row_pos;
+        w = (M.w == 0 || (M.f > 0 && idr >= M.max_id - M.f)) ? 0x7fffffff : M.w;
+        lo = idr - w;
+        ctx = M.c > 0 && idr == 0;
+    }
+    __device__ __forceinline__ bool valid(const SeqMask& M, int key_pos) const {
+        const int ids = M.id(key_pos);
+        return (key_pos == pos) | ((unsigned)(ids - lo) < (unsigned)w) | (ctx & (ids < M.max_id));
+    }
+};
+
+// P^T for one 32x32 block of S^T: p = s * sigmoid(alpha s) = s * rcp(1 + exp2(c1 s)), c1 = -alpha log2(e),
+// zeroed where the mask says so, rounded to the 16-bit type and packed as two MFMA B operands.
+// `sp0` is the sequence position of this lane's first kv slot of the block.
+template <class TT, bool MASKED>
+__device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], float c1, const SeqMask& M,
+                                          const RowMask& row, int sp0) {
+    typedef typename TT::elem elem;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        // eight elements at a time, fenced, so that the scheduler cannot pile up temporaries of all sixteen
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int r = half * 8 + j;
+            float x = s[r];
+            float e = __builtin_amdgcn_exp2f(x * c1);
+            float pr = x * __builtin_amdgcn_rcpf(1.0f + e);
+            if (MASKED) pr = row.valid(M, sp0 + 8 * (r >> 2) + (r & 3)) ? pr : 0.f;
+            pb[half][j] = (elem)pr;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+// B operand of the first product for one block of 32 query rows: lane holds Q[row][16 ks + 8 g .. +8).
+// Rows at or past `nq` re-read the last valid row (their outputs are never stored).
+template <class TT, int KS>
+__device__ __forceinline__ void load_q_operand(typename TT::vec8 (&qreg)[KS], const char* q, int64_t qrow0, int ql, int nq,
+                                               int64_t q_rs, int64_t q_hs, int h, int g) {
+    typedef typename TT::vec8 vec8;
+    ql = ql < nq ? ql : nq - 1;
+    const char* qp = q + ((qrow0 + ql) * q_rs + (int64_t)h * q_hs) * 2 + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const vec8*)(qp + ks * 32);
+}
+
+// Byte offsets, inside a K tile and a V tile, of this lane's LDS reads; constant over the kv loop.
+// K (A operand of the first product): row sub*32 + lane%32, logical chunk 2 ks + lane/32.
+// V^T (A operand of the second product) through ds_read_b64_tr_b16: within each group of 16 lanes,
+// lane 4j+q supplies the address of 4 consecutive dv of kv row j and the hardware hands lane i the four
+// kv rows of dv i.  Operand lane l must end up with dv = l%32 and kv slots {4g..4g+3} (first read) and
+// {8+4g..8+4g+3} (second read), g = l/32 -- the order in which the accumulator of the first product
+// holds its kv rows.
+template <int DQK, int DV>
+__device__ __forceinline__ void lds_read_offsets(int (&kaddr)[DQK / 16], int (&vaddr)[2][DV / 32], int lane) {
+    constexpr int KS = DQK / 16, DT = DV / 32, KROW = DQK * 2, VROW = DV * 2, KCH = DQK / 8, VCH = DV / 8;
+    const int g = lane >> 5, l32 = lane & 31;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = l32 * KROW + (((2 * ks + g) ^ swz_k<KCH>(l32)) * 16);
+    const int i16 = lane & 15, half = (lane >> 4) & 1;
+    const int jrow = i16 >> 2, q4 = i16 & 3;
+#pragma unroll
+    for (int sec = 0; sec < 2; ++sec) {
+        const int row = 8 * sec + 4 * g + jrow;  // + 32 sub + 16 t
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int chunk = dt * 4 + 2 * half + (q4 >> 1);
+            vaddr[sec][dt] = row * VROW + ((chunk ^ swz_v<VCH>(row)) * 16) + (q4 & 1) * 8;
+        }
+    }
+}
+
+// A operand of the second product (32 dv x 16 kv) from two transposing LDS reads.
+template <class TT>
+__device__ __forceinline__ typename TT::vec8 read_vt_operand(const char* lo_addr, const char* hi_addr) {
+    s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, lo_addr));
+    s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, hi_addr));
+    s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(typename TT::vec8, both);
+}
+
+// out[q, dv] = oscale * O^T[dv, q] for one block of 32 query rows; the lane holds 4 consecutive dv per
+// (dv tile, r/4), stored as 8 bytes.  QT is deduced from the accumulator array.
+template <class TT, int DT, int QT>
+__device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int qt, char* o, int64_t orow0, int ql, int nq,
+                                             int64_t o_rs, int64_t o_hs, int h, int g, float oscale) {
+    typedef typename TT::elem elem;
+    typedef __attribute__((ext_vector_type(4))) elem elem4;
+    if (ql >= nq) return;
+    char* op = o + ((orow0 + ql) * o_rs + (int64_t)h * o_hs) * 2 + g * 8;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            elem4 o4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o4[i] = (elem)(oacc[dt][qt][r4 * 4 + i] * oscale);
+            *(elem4*)(op + (dt * 32 + r4 * 8) * 2) = o4;
+        }
+}
+
+// Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit
+// per-lane byte offset, so that issuing a copy costs no vector arithmetic.
+__device__ __forceinline__ void global_load_lds16_soff(const char* base_uniform, unsigned lane_offset, const char* lds_base) {
+    const unsigned m0 = (unsigned)(uintptr_t)HSTU_LDS(const char, lds_base);
+    const uint64_t sbase = (uint64_t)uniform64((int64_t)(uintptr_t)base_uniform);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(m0), "v"(lane_offset), "s"(sbase)
+                 : "memory");
+}
+
+// Copy `ROWS` rows of `ROWBYTES` bytes from global memory into LDS with the chunk swizzle.
+// Rows at or beyond `n_rows_valid` re-read the last valid row (their products are masked).
+template <int ROWS, int ROWBYTES, int NTHREADS, bool IS_V>
+__device__ __forceinline__ void load_tile_to_lds(const char* gbase, int64_t row_stride_bytes, int row0,
+                                                 int last_row, char* lds_tile, int wave, int lane) {
+    constexpr int CH = ROWBYTES / 16;                // 16-byte chunks per row
+    constexpr int INSTR = ROWS * CH / 64;            // wave-wide copies per tile
+    constexpr int NWAVES = NTHREADS / 64;
+    static_assert(INSTR % NWAVES == 0, "tile copy must split evenly over the waves");
+#pragma unroll
+    for (int i = 0; i < INSTR / NWAVES; ++i) {
+        int inst = wave + i * NWAVES;
+        int p = inst * 64 + lane;
+        int row = p / CH;
+        int phys = p % CH;
+        int logical = phys ^ (IS_V ? swz_v<CH>(row) : swz_k<CH>(row));
+        int grow = row0 + row;
+        grow = grow > last_row ? last_row : grow;
+        const char* src = gbase + (int64_t)grow * row_stride_bytes + logical * 16;
+        global_load_lds16(src, lds_tile + inst * 1024);
+    }
+}
+
+}  // namespace hstu

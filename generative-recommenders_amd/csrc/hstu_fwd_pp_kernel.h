@@ -1,0 +1,337 @@
+// Ping-pong forward kernel for long sequences: 8 waves per workgroup, 256 query rows, one workgroup per CU.
+//
+// Per score element the matrix cores need 512 flops (half a cycle per element and SIMD at peak) while
+// s*sigmoid(alpha s) needs about 30 VALU issue cycles per 64 elements -- the two cost the same, and a wave
+// that has just issued an MFMA cannot issue VALU work for a while, so the two kinds of work must come from
+// different waves of a SIMD at the same time.  The two waves that share a SIMD are therefore kept in
+// opposite phases on purpose: waves 0-3 ("A") run the matrix phase of a kv tile (O^T += V^T P^T of the
+// previous tile interleaved with S^T = K Q^T of this one) while waves 4-7 ("B") run the VALU phase
+// (P^T from S^T) of the tile before; a workgroup barrier swaps the roles.  Every tile takes two phases;
+// B trails A by one phase.
+//
+// The matrix phase is one straight line of MFMAs whose LDS operands are requested PD MFMAs ahead
+// (rotating registers, order pinned with sched_barrier) so that one wave alone keeps its matrix core fed.
+// Tiles are never skipped per wave: a tile with nothing valid for a wave's rows just gets P^T = 0.
+//
+// LDS holds three K tiles and three V tiles.  In step i the copies of V(i+1) and K(i+2) are issued from
+// inside the matrix phase (spread between MFMAs; their slots were last read in step i-1), and the end of
+// step i waits only for the copies issued in step i-1, so each copy has three to four phases to land.
+// The scheme common to all kernels is described at the top of hstu_common.h.
+#pragma once
+#include <type_traits>
+
+#include "hstu_common.h"
+
+namespace hstu {
+
+// Direct HBM -> LDS copy of one tile, spread over 8 waves; per-lane byte offsets from the tile's first row
+// are precomputed.
+template <int ROWS, int ROWBYTES, bool IS_V>
+struct TileCopy {
+    static constexpr int CH = ROWBYTES / 16;
+    static constexpr int NI = ROWS * CH / 64;       // wave-wide copy instructions per tile
+    static constexpr int PER_WAVE = (NI + 7) / 8;
+    unsigned off[PER_WAVE];       // for a tile that lies entirely inside the sequence
+    unsigned off_last[PER_WAVE];  // for the sequence's last, partly filled tile: rows past the end re-read the last row
+    static __device__ __forceinline__ unsigned lane_offset(int inst, int lane, int64_t row_stride_bytes, int max_row) {
+        const int p = inst * 64 + lane;
+        int row = p / CH;
+        const int phys = p % CH;
+        const int logical = phys ^ (IS_V ? swz_v<CH>(row) : swz_k<CH>(row));
+        row = row < max_row ? row : max_row;
+        return (unsigned)(row * row_stride_bytes) + logical * 16;
+    }
+    __device__ __forceinline__ void init(int wave, int lane, int64_t row_stride_bytes, int n) {
+        const int last_valid = (n - 1) % ROWS;  // last filled row of the sequence's last tile
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) {
+            off[i] = lane_offset(wave + 8 * i, lane, row_stride_bytes, ROWS);
+            off_last[i] = lane_offset(wave + 8 * i, lane, row_stride_bytes, last_valid);
+        }
+    }
+    // Copy instruction `i` (0 .. PER_WAVE-1) of this wave for the tile starting at row `row0`;
+    // `gbase` points at row 0 of the sequence for this head.
+    __device__ __forceinline__ void issue_one(int i, const char* gbase, int64_t row_stride_bytes, int row0, int n,
+                                              char* lds_tile, int wave) const {
+        const int inst = wave + 8 * i;
+        if (inst < NI) {
+            const char* tile_base = gbase + (int64_t)row0 * row_stride_bytes;  // wave-uniform
+            const unsigned o = (row0 + ROWS > n) ? off_last[i] : off[i];
+            global_load_lds16_soff(tile_base, o, lds_tile + inst * 1024);
+        }
+    }
+    __device__ __forceinline__ void issue(const char* gbase, int64_t row_stride_bytes, int row0, int n, char* lds_tile,
+                                          int wave) const {
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; ++i) issue_one(i, gbase, row_stride_bytes, row0, n, lds_tile, wave);
+    }
+};
+
+template <class TT, int DQK, int DV, int BN>
+__global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) {
+    typedef typename TT::vec8 vec8;
+    static_assert(DQK == DV, "the interleaved matrix phase assumes as many first-product as second-product MFMAs");
+    constexpr int BM = 256;
+    constexpr int NS = BN / 32;
+    constexpr int KS = DQK / 16;
+    constexpr int DT = DV / 32;
+    constexpr int KROW = DQK * 2, VROW = DV * 2;
+    constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
+    constexpr int NSLOT = 3;
+    // LDS: 3 K slots, then 3 V slots.  A static array (the only LDS object, so it sits at address 0) lets
+    // every tile and slot offset fold into the immediate field of the LDS reads.
+    __shared__ __attribute__((aligned(1024))) char smem[NSLOT * (KTILE + VTILE)];
+    constexpr int VOFF = NSLOT * KTILE;
+    // The immediate offset of an LDS read reaches 64 KB.  K reads stay below that; V reads go through address
+    // registers biased by VBIAS so that VOFF - VBIAS + slot and tile offsets fit the immediate as well.
+    constexpr int VBIAS = (NSLOT * (KTILE + VTILE) > 65536) ? 32768 : 0;
+    static_assert(VOFF >= VBIAS && VOFF - VBIAS + NSLOT * VTILE <= 65536 && NSLOT * KTILE <= 65536, "LDS immediates");
+    constexpr int NOPS = NS * KS + NS * 2 * DT;   // MFMAs of one matrix phase
+    constexpr int PD = NOPS >= 16 ? 6 : 4;        // operands in flight
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = wave >> 2;    // 0: waves 0-3 (A), 1: waves 4-7 (B); waves w and w+4 share a SIMD
+    const int g = lane >> 5;
+    const int l32 = lane & 31;
+
+    Work W;
+    if (!decode_work<BM, BN>(p, W)) return;
+    const SeqMask& M = W.M;
+    const int n = W.n, nq = W.nq;
+
+    const int wq0 = W.m0 + wave * 32;
+    const int wR0 = W.rbase + wq0;
+    const int wR1 = (wq0 + 32 < nq ? W.rbase + wq0 + 32 : W.rbase + nq) - 1;
+
+    // Tiles [full_begin, full_end) are valid in every element for this wave's rows (no mask code): the tile
+    // lies strictly before the first row's id and inside every row's window.  Every other tile takes the
+    // exact per-element predicate, and so does a sequence that breaks the caller contract
+    // "non-target positions >= contextual_seq_len" (ids would go negative).
+    int full_begin = 0, full_end = 0;
+    if (wR1 >= wR0 && W.u >= p.c && W.u >= 0) {
+        const int idr_lo = M.id(wR0), idr_hi = M.id(wR1);
+        full_end = (idr_lo + M.shift) / BN;          // keys s with s - shift < id(first row)
+        if (full_end * BN > n) full_end = n / BN;
+        if (p.w > 0 && idr_hi - p.w > 0) full_begin = (idr_hi - p.w + M.shift + BN - 1) / BN;
+    }
+
+    // This kernel walks the contiguous tile range [jt_begin, jt_end): a tile inside it that holds no valid
+    // pair (other targets' columns of a target row block) is computed and masked to zero rather than
+    // skipped, which keeps the step count known up front and the loop free of side exits.
+    const int jt_end = W.jt_end;
+    const int T = jt_end - W.jt_begin;  // steps
+    if (T <= 0) return;  // cannot happen for a row block with rows (each row sees itself); kept for safety
+    int t_cur = W.jt_begin;
+
+    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * 2;
+    const char* vbase = p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * 2;
+    const int64_t k_rsb = p.k_rs * 2, v_rsb = p.v_rs * 2;
+    typedef TileCopy<BN, KROW, false> KCopy;
+    typedef TileCopy<BN, VROW, true> VCopy;
+    KCopy kcopy;
+    VCopy vcopy;
+    kcopy.init(wave, lane, k_rsb, n);
+    vcopy.init(wave, lane, v_rsb, n);
+    constexpr int NPW = KCopy::PER_WAVE + VCopy::PER_WAVE;  // copy instructions per wave and step
+    static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
+
+    // before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1
+    kcopy.issue(kbase, k_rsb, t_cur * BN, n, smem, wave);
+    vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
+    kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
+
+    vec8 qreg[KS];
+    const int64_t qrow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
+    load_q_operand<TT, KS>(qreg, p.q, qrow0, wq0 + l32, nq, p.q_rs, p.q_hs, W.h, g);
+    RowMask row;
+    row.init(M, wR0 + l32);
+
+    int kaddr[KS];
+    int vaddr[2][DT];
+    lds_read_offsets<DQK, DV>(kaddr, vaddr, lane);
+#pragma unroll
+    for (int sec = 0; sec < 2; ++sec)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            vaddr[sec][dt] += VBIAS;
+            asm volatile("" : "+v"(vaddr[sec][dt]));  // keep the bias in the register, out of the immediates
+        }
+
+    f32x16_t oacc[DT][1];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[dt][0][r] = 0.f;
+
+    f32x16_t s[NS];        // S^T of the tile in flight between this wave's matrix and VALU phases
+    vec8 pb[NS][2];        // P^T of the tile in flight between its VALU phase and its next matrix phase
+
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+
+    // ---- building blocks ------------------------------------------------------------------------------
+    // Copy instruction j (0 .. NPW-1) of the step of list entry i (SLOT = i % 3): the V tile of entry i+1,
+    // then the K tile of entry i+2.  Past the end of the list the last entry is copied again (redundant, but
+    // it keeps the number of copy instructions per step, and with it the vmcnt arithmetic, constant).
+    auto issue_copy = [&](auto slot_c, int j) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        const int tv = t_cur + 1 < jt_end ? t_cur + 1 : jt_end - 1;
+        const int tk = t_cur + 2 < jt_end ? t_cur + 2 : jt_end - 1;
+        if (j < VCopy::PER_WAVE)
+            vcopy.issue_one(j, vbase, v_rsb, tv * BN, n, smem + VOFF + ((SLOT + 1) % NSLOT) * VTILE, wave);
+        else
+            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, n, smem + ((SLOT + 2) % NSLOT) * KTILE, wave);
+    };
+    // S^T = K Q^T only (first step), K slot chosen at run time.
+    auto gemm1_only = [&](int kslot) __attribute__((always_inline)) {
+        const char* kt = smem + kslot * KTILE;
+#pragma unroll
+        for (int sub = 0; sub < NS; ++sub) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[sub][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                vec8 a = *HSTU_LDS(const vec8, kt + sub * 32 * KROW + kaddr[ks]);
+                s[sub] = TT::mfma(a, qreg[ks], s[sub]);
+            }
+        }
+    };
+    // O^T += V^T P^T only (after the last step), V slot chosen at run time.
+    auto gemm2_only = [&](int vslot) __attribute__((always_inline)) {
+        const char* vt = smem + (VOFF - VBIAS) + vslot * VTILE;
+#pragma unroll
+        for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const char* vb = vt + (sub * 32 + tt * 16) * VROW;
+                    vec8 a = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+                    oacc[dt][0] = TT::mfma(a, pb[sub][tt], oacc[dt][0]);
+                }
+    };
+    // Full matrix phase of list entry i (SLOT = i % 3): second product of entry i-1 interleaved with the
+    // first product of entry i, plus this wave's share of the step's copies.
+    // MFMA k: even k -> second product (sub, tt, dt) = ((k/2)/(2 DT), ((k/2)/DT) % 2, (k/2) % DT);
+    //         odd k  -> first product  (ks, sub) = ((k/2)/NS, (k/2) % NS).
+    auto matrix_phase = [&](auto slot_c) __attribute__((always_inline)) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        const char* kt = smem + SLOT * KTILE;
+        const char* vt = smem + (VOFF - VBIAS) + ((SLOT + 2) % NSLOT) * VTILE;
+        auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
+            const int o = k >> 1;
+            if ((k & 1) == 0) {
+                const int sub = o / (2 * DT), tt = (o / DT) % 2, dt = o % DT;
+                const char* vb = vt + (sub * 32 + tt * 16) * VROW;
+                return read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+            } else {
+                const int ks = o / NS, sub = o % NS;
+                return *HSTU_LDS(const vec8, kt + sub * 32 * KROW + kaddr[ks]);
+            }
+        };
+#pragma unroll
+        for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[sub][r] = 0.f;
+        vec8 fr[PD];
+#pragma unroll
+        for (int k = 0; k < PD; ++k) fr[k] = load_op(k);
+#pragma unroll
+        for (int k = 0; k < NOPS; ++k) {
+            __builtin_amdgcn_sched_barrier(0);
+            const int o = k >> 1;
+            if ((k & 1) == 0) {
+                const int sub = o / (2 * DT), tt = (o / DT) % 2, dt = o % DT;
+                oacc[dt][0] = TT::mfma(fr[k % PD], pb[sub][tt], oacc[dt][0]);
+            } else {
+                const int ks = o / NS, sub = o % NS;
+                s[sub] = TT::mfma(fr[k % PD], qreg[ks], s[sub]);
+            }
+            if (k + PD < NOPS) fr[k % PD] = load_op(k + PD);
+            // spread the copies over the phase: one after every (NOPS/NPW)-th MFMA
+            if (k % (NOPS / NPW) == 1) issue_copy(slot_c, k / (NOPS / NPW));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // VALU phase: P^T from S^T of `tile`.
+    auto valu_phase = [&](int tile) __attribute__((always_inline)) {
+        if (tile >= full_begin && tile < full_end) {
+#pragma unroll
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, false>(s[sub], pb[sub], p.c1, M, row, 0);
+        } else {
+#pragma unroll
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, true>(s[sub], pb[sub], p.c1, M, row, tile * BN + 4 * g + sub * 32);
+        }
+    };
+    auto end_of_step = [&]() __attribute__((always_inline)) {
+        // every copy but this step's has landed for this wave ...
+        __builtin_amdgcn_s_waitcnt((NPW & 0xF) | ((NPW >> 4) << 14) | 0x0F70);
+        __syncthreads();  // ... and for every wave
+    };
+    typedef std::integral_constant<int, 0> S0;
+    typedef std::integral_constant<int, 1> S1;
+    typedef std::integral_constant<int, 2> S2;
+
+    // Both groups execute the same barriers: two per step and one in the drain.  Step i uses slot i % 3;
+    // step 0 is peeled (first product only), then whole rounds of three steps, then the remainder.
+    const int rounds = (T - 1) / 3, rem = (T - 1) % 3;
+    if (grp == 0) {
+        // ---- A: [matrix(i) | VALU(i)] per step
+        auto stepA = [&](auto slot_c) __attribute__((always_inline)) {
+            matrix_phase(slot_c);
+            __syncthreads();
+            valu_phase(t_cur);
+            end_of_step();
+            ++t_cur;
+        };
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
+        gemm1_only(0);
+        __syncthreads();
+        valu_phase(t_cur);
+        end_of_step();
+        ++t_cur;
+        for (int r = 0; r < rounds; ++r) {
+            stepA(S1{});
+            stepA(S2{});
+            stepA(S0{});
+        }
+        if (rem >= 1) stepA(S1{});
+        if (rem >= 2) stepA(S2{});
+        gemm2_only((T - 1) % NSLOT);
+        __syncthreads();
+    } else {
+        // ---- B: [VALU(i-1) | matrix(i)] per step, one phase behind A
+        auto stepB = [&](auto slot_c) __attribute__((always_inline)) {
+            valu_phase(t_cur - 1);
+            __syncthreads();
+            matrix_phase(slot_c);
+            end_of_step();
+            ++t_cur;
+        };
+#pragma unroll
+        for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
+        __syncthreads();
+        gemm1_only(0);
+        end_of_step();
+        ++t_cur;
+        for (int r = 0; r < rounds; ++r) {
+            stepB(S1{});
+            stepB(S2{});
+            stepB(S0{});
+        }
+        if (rem >= 1) stepB(S1{});
+        if (rem >= 2) stepB(S2{});
+        valu_phase(t_cur - 1);
+        __syncthreads();
+        gemm2_only((T - 1) % NSLOT);
+    }
+    // the redundant copies of the last steps may still be in flight: they must land before the LDS is released
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+    const int64_t orow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
+    store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
+}
+
+}  // namespace hstu
