@@ -184,7 +184,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     p.c = a->contextual_seq_len;
     p.f = a->min_full_attn_seq_len;
     p.c1 = -a->alpha * 1.4426950408889634f;
-    p.oscale = a->alpha / (float)a->max_seq_len;
+    p.oscale = a->alpha == 0.0f ? 0.0f : -1.0f / ((float)a->max_seq_len * 1.4426950408889634f);
 
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long num_pairs_ll = (long long)a->batch * a->heads;

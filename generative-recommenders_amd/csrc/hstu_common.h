@@ -62,8 +62,8 @@ struct FwdParams {
     int max_seq_len;
     int delta;          // 0 = full attention
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
-    float c1;           // -alpha * log2(e)
-    float oscale;       // alpha / max_seq_len
+    float c1;           // -alpha * log2(e): Q is multiplied by it when loaded
+    float oscale;       // (alpha / max_seq_len) / c1 = -1 / (max_seq_len * log2(e)); 0 if alpha == 0
 };
 
 struct Bf16 {
@@ -247,11 +247,13 @@ struct RowMask {
     }
 };
 
-// P^T for one 32x32 block of S^T: p = s * sigmoid(alpha s) = s * rcp(1 + exp2(c1 s)), c1 = -alpha log2(e),
-// zeroed where the mask says so, rounded to the 16-bit type and packed as two MFMA B operands.
+// P^T for one 32x32 block.  The accumulator holds t = c1*s with c1 = -alpha*log2(e) (Q was pre-scaled), so
+// s*sigmoid(alpha s) = (t / c1) * rcp(1 + exp2(t)); the kernel forms p = t * rcp(1 + exp2(t)) and leaves the
+// constant 1/c1 to the output scale.  p is zeroed where the mask says so, rounded to the 16-bit type and
+// packed as two MFMA B operands.
 // `sp0` is the sequence position of this lane's first kv slot of the block.
 template <class TT, bool MASKED>
-__device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], float c1, const SeqMask& M,
+__device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], const SeqMask& M,
                                           const RowMask& row, int sp0) {
     typedef typename TT::elem elem;
 #pragma unroll
@@ -261,7 +263,7 @@ __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (
         for (int j = 0; j < 8; ++j) {
             const int r = half * 8 + j;
             float x = s[r];
-            float e = __builtin_amdgcn_exp2f(x * c1);
+            float e = __builtin_amdgcn_exp2f(x);
             float pr = x * __builtin_amdgcn_rcpf(1.0f + e);
             if (MASKED) pr = row.valid(M, sp0 + 8 * (r >> 2) + (r & 3)) ? pr : 0.f;
             pb[half][j] = (elem)pr;
@@ -270,16 +272,26 @@ __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (
     }
 }
 
-// B operand of the first product for one block of 32 query rows: lane holds Q[row][16 ks + 8 g .. +8).
-// Rows at or past `nq` re-read the last valid row (their outputs are never stored).
+// B operand of the first product for one block of 32 query rows: lane holds Q[row][16 ks + 8 g .. +8),
+// multiplied by `qscale` = -alpha*log2(e) and rounded back to the 16-bit type, so that the first product
+// directly yields t = -alpha*log2(e)*s, the argument of the exp2 in the sigmoid; this removes one VALU
+// multiply per score element, which is what the kernel is short of.  The extra rounding of Q is of the size
+// of the rounding the 16-bit inputs already carry.  Rows at or past `nq` re-read the last valid row (their
+// outputs are never stored).
 template <class TT, int KS>
 __device__ __forceinline__ void load_q_operand(typename TT::vec8 (&qreg)[KS], const char* q, int64_t qrow0, int ql, int nq,
-                                               int64_t q_rs, int64_t q_hs, int h, int g) {
+                                               int64_t q_rs, int64_t q_hs, int h, int g, float qscale) {
     typedef typename TT::vec8 vec8;
+    typedef typename TT::elem elem;
     ql = ql < nq ? ql : nq - 1;
     const char* qp = q + ((qrow0 + ql) * q_rs + (int64_t)h * q_hs) * 2 + g * 16;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qreg[ks] = *(const vec8*)(qp + ks * 32);
+    for (int ks = 0; ks < KS; ++ks) {
+        vec8 raw = *(const vec8*)(qp + ks * 32);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) raw[j] = (elem)((float)raw[j] * qscale);
+        qreg[ks] = raw;
+    }
 }
 
 // Byte offsets, inside a K tile and a V tile, of this lane's LDS reads; constant over the kv loop.

@@ -12,7 +12,7 @@ namespace hstu {
 template <class TT, int DQK, int DV, int QT, int BN, bool MASKED>
 __device__ __forceinline__ void tile_compute(const char* kt, const char* vt, const typename TT::vec8 (&qreg)[QT][DQK / 16],
                                              f32x16_t (&oacc)[DV / 32][QT], const int (&kaddr)[DQK / 16],
-                                             const int (&vaddr)[2][DV / 32], float c1, const SeqMask& M, int sp0,
+                                             const int (&vaddr)[2][DV / 32], const SeqMask& M, int sp0,
                                              const RowMask (&rows)[QT]) {
     typedef typename TT::vec8 vec8;
     constexpr int NS = BN / 32, KS = DQK / 16, DT = DV / 32, KROW = DQK * 2, VROW = DV * 2;
@@ -36,7 +36,7 @@ __device__ __forceinline__ void tile_compute(const char* kt, const char* vt, con
 #pragma unroll
     for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) silu_pack<TT, MASKED>(s[sub][qt], pb[sub][qt], c1, M, rows[qt], sp0 + sub * 32);
+        for (int qt = 0; qt < QT; ++qt) silu_pack<TT, MASKED>(s[sub][qt], pb[sub][qt], M, rows[qt], sp0 + sub * 32);
     // ---- O^T += V^T P^T
 #pragma unroll
     for (int sub = 0; sub < NS; ++sub)
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     vec8 qreg[QT][KS];
     const int64_t qrow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) load_q_operand<TT, KS>(qreg[qt], p.q, qrow0, wq0 + qt * 32 + l32, nq, p.q_rs, p.q_hs, W.h, g);
+    for (int qt = 0; qt < QT; ++qt) load_q_operand<TT, KS>(qreg[qt], p.q, qrow0, wq0 + qt * 32 + l32, nq, p.q_rs, p.q_hs, W.h, g, p.c1);
 
     RowMask rows[QT];
 #pragma unroll
@@ -125,9 +125,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
         const int cls = M.classify(wR0, wR1, jt * BN, BN);
         const char* kt = smem + stage * STAGE;
         if (cls == 2) {
-            tile_compute<TT, DQK, DV, QT, BN, false>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
+            tile_compute<TT, DQK, DV, QT, BN, false>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, M, jt * BN + 4 * g, rows);
         } else if (cls == 1) {
-            tile_compute<TT, DQK, DV, QT, BN, true>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
+            tile_compute<TT, DQK, DV, QT, BN, true>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, M, jt * BN + 4 * g, rows);
         }
         jt = jn;
         stage ^= 1;

@@ -24,13 +24,15 @@
 
 namespace hstu {
 
-// Direct HBM -> LDS copy of one tile, spread over 8 waves; per-lane byte offsets from the tile's first row
-// are precomputed.
+// Direct HBM -> LDS copy of one tile, spread over the four "A" waves (copies issued from the "B" waves'
+// matrix phase were measured to stall it; from the A waves they are free); per-lane byte offsets from the
+// tile's first row are precomputed.
 template <int ROWS, int ROWBYTES, bool IS_V>
 struct TileCopy {
     static constexpr int CH = ROWBYTES / 16;
     static constexpr int NI = ROWS * CH / 64;       // wave-wide copy instructions per tile
-    static constexpr int PER_WAVE = (NI + 7) / 8;
+    static constexpr int NCW = 4;                   // waves that issue copies
+    static constexpr int PER_WAVE = (NI + NCW - 1) / NCW;
     unsigned off[PER_WAVE];       // for a tile that lies entirely inside the sequence
     unsigned off_last[PER_WAVE];  // for the sequence's last, partly filled tile: rows past the end re-read the last row
     static __device__ __forceinline__ unsigned lane_offset(int inst, int lane, int64_t row_stride_bytes, int max_row) {
@@ -45,15 +47,15 @@ struct TileCopy {
         const int last_valid = (n - 1) % ROWS;  // last filled row of the sequence's last tile
 #pragma unroll
         for (int i = 0; i < PER_WAVE; ++i) {
-            off[i] = lane_offset(wave + 8 * i, lane, row_stride_bytes, ROWS);
-            off_last[i] = lane_offset(wave + 8 * i, lane, row_stride_bytes, last_valid);
+            off[i] = lane_offset(wave + NCW * i, lane, row_stride_bytes, ROWS);
+            off_last[i] = lane_offset(wave + NCW * i, lane, row_stride_bytes, last_valid);
         }
     }
     // Copy instruction `i` (0 .. PER_WAVE-1) of this wave for the tile starting at row `row0`;
     // `gbase` points at row 0 of the sequence for this head.
     __device__ __forceinline__ void issue_one(int i, const char* gbase, int64_t row_stride_bytes, int row0, int n,
                                               char* lds_tile, int wave) const {
-        const int inst = wave + 8 * i;
+        const int inst = wave + NCW * i;
         if (inst < NI) {
             const char* tile_base = gbase + (int64_t)row0 * row_stride_bytes;  // wave-uniform
             const unsigned o = (row0 + ROWS > n) ? off_last[i] : off[i];
@@ -137,13 +139,15 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
 
     // before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1
-    kcopy.issue(kbase, k_rsb, t_cur * BN, n, smem, wave);
-    vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
-    kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
+    if (grp == 0) {
+        kcopy.issue(kbase, k_rsb, t_cur * BN, n, smem, wave);
+        vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
+        kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
+    }
 
     vec8 qreg[KS];
     const int64_t qrow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
-    load_q_operand<TT, KS>(qreg, p.q, qrow0, wq0 + l32, nq, p.q_rs, p.q_hs, W.h, g);
+    load_q_operand<TT, KS>(qreg, p.q, qrow0, wq0 + l32, nq, p.q_rs, p.q_hs, W.h, g, p.c1);
     RowMask row;
     row.init(M, wR0 + l32);
 
@@ -176,6 +180,7 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     // it keeps the number of copy instructions per step, and with it the vmcnt arithmetic, constant).
     auto issue_copy = [&](auto slot_c, int j) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
+        if (grp != 0) return;
         const int tv = t_cur + 1 < jt_end ? t_cur + 1 : jt_end - 1;
         const int tk = t_cur + 2 < jt_end ? t_cur + 2 : jt_end - 1;
         if (j < VCopy::PER_WAVE)
@@ -258,10 +263,10 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     auto valu_phase = [&](int tile) __attribute__((always_inline)) {
         if (tile >= full_begin && tile < full_end) {
 #pragma unroll
-            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, false>(s[sub], pb[sub], p.c1, M, row, 0);
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, false>(s[sub], pb[sub], M, row, 0);
         } else {
 #pragma unroll
-            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, true>(s[sub], pb[sub], p.c1, M, row, tile * BN + 4 * g + sub * 32);
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, true>(s[sub], pb[sub], M, row, tile * BN + 4 * g + sub * 32);
         }
     };
     auto end_of_step = [&]() __attribute__((always_inline)) {
