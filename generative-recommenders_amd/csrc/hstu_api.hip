@@ -190,8 +190,10 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     const long long num_pairs_ll = (long long)a->batch * a->heads;
     if (num_pairs_ll > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     const int num_pairs = (int)num_pairs_ll;
+    // Automatic choice: the ping-pong kernel (256-row blocks, one workgroup per CU) wins once sequences
+    // are long enough to keep its pipeline full; short sequences waste less in 128-row blocks.
     int cfg = a->tile_config;
-    if (cfg == 0) cfg = 1;
+    if (cfg == 0) cfg = a->max_seq_len >= 2048 ? 2 : 1;
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
     return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
 }

@@ -160,7 +160,7 @@ struct Work {
 };
 
 // Decode blockIdx.x.  Workgroup ids go round-robin over the 8 XCDs, so ids congruent mod 8 share
-// an L2: all row blocks of one (sequence, head) pair stay on one XCD, heaviest (last) block first.
+// an L2: all row blocks of one (sequence, head) pair stay on one XCD, heaviest block first.
 // Returns false if this workgroup has nothing to do.
 template <int BM, int BN>
 __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
@@ -169,7 +169,10 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
     const int slot = bid >> 3;
     const int pair = (slot / p.num_mb) * 8 + xcd;
     if (pair >= p.B * p.H) return false;
-    const int mb = p.num_mb - 1 - (slot % p.num_mb);
+    // heaviest row block first: the last one -- except that with a contextual prefix the first row block
+    // (its contextual rows see every non-target key) is the heaviest of all
+    const int rank = slot % p.num_mb;
+    const int mb = p.c > 0 ? (rank == 0 ? 0 : p.num_mb - rank) : p.num_mb - 1 - rank;
     w.b = pair / p.H;
     w.h = pair - w.b * p.H;
     int64_t seq_start, seq_end;
