@@ -32,7 +32,7 @@ constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 template <class TT, int DQK, int DV, int QT, int NW, int BN, int OCC>
 int launch(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
     constexpr int BM = NW * QT * 32;
-    constexpr int smem = 2 * BN * (DQK + DV) * 2;
+    constexpr int smem = 2 * BN * (DQK + DV) * TT::ES;
     auto kern = hstu::hstu_fwd_kernel<TT, DQK, DV, QT, NW, BN, OCC>;
     static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; racing threads set the same value
     if (!attr_done) {
@@ -110,7 +110,7 @@ const char* hstu_hip_status_string(int status) {
         case HSTU_ERR_BAD_DTYPE: return "only bf16, fp16 and fp8_e4m3 data types are supported";
         case HSTU_ERR_BAD_HEAD_DIM: return "unsupported head dimension (built: dqk == dv in {32, 64, 128})";
         case HSTU_ERR_MISALIGNED:
-            return "q/k/v/out must be 16-byte aligned with row and head strides that are multiples of 8 elements";
+            return "q/k/v/out must be 16-byte aligned with row and head strides that are multiples of 16 bytes";
         case HSTU_ERR_BAD_SHAPE: return "inconsistent sizes";
         case HSTU_ERR_UNSUPPORTED: return "argument combination not built";
         case HSTU_ERR_LAUNCH: return "HIP launch failed";
@@ -142,12 +142,13 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     if (a->dqk != 32 && a->dqk != 64 && a->dqk != 128) return HSTU_ERR_BAD_HEAD_DIM;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;  // nothing to do; pointers may be anything
     if (!a->q || !a->k || !a->v || !a->out || !a->seq_offsets) return HSTU_ERR_NULL_POINTER;
-    if (a->dtype == HSTU_FP8_E4M3) return HSTU_ERR_UNSUPPORTED;
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out)) return HSTU_ERR_MISALIGNED;
     const int64_t strides[8] = {a->q_row_stride, a->q_head_stride, a->k_row_stride, a->k_head_stride,
                                 a->v_row_stride, a->v_head_stride, a->o_row_stride, a->o_head_stride};
+    // rows of q/k/v start on 16-byte boundaries: 8 elements of 16 bits, 16 of 8 bits; the output is always 16 bit
+    const int64_t in_mask = a->dtype == HSTU_FP8_E4M3 ? 15 : 7;
     for (int i = 0; i < 8; ++i)
-        if (strides[i] < 0 || (strides[i] & 7) != 0) return HSTU_ERR_MISALIGNED;
+        if (strides[i] < 0 || (strides[i] & (i < 6 ? in_mask : 7)) != 0) return HSTU_ERR_MISALIGNED;
     return HSTU_OK;
 }
 
@@ -185,6 +186,12 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     p.f = a->min_full_attn_seq_len;
     p.c1 = -a->alpha * 1.4426950408889634f;
     p.oscale = a->alpha == 0.0f ? 0.0f : -1.0f / ((float)a->max_seq_len * 1.4426950408889634f);
+    if (a->dtype == HSTU_FP8_E4M3) {
+        // real value = stored value * scale: the score scales go into c1 (applied to the accumulator), the
+        // value scale and the factor P is stored with go into the output scale
+        p.c1 *= a->q_scale * a->k_scale;
+        p.oscale *= a->v_scale / hstu::Fp8::PSCALE;
+    }
 
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long num_pairs_ll = (long long)a->batch * a->heads;
@@ -195,7 +202,8 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     int cfg = a->tile_config;
     if (cfg == 0) cfg = a->max_seq_len >= 2048 ? 2 : 1;
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
-    return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
+    if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
+    return launch_dim<hstu::Fp8>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
 }
 
 }  // extern "C"

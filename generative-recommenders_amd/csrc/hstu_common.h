@@ -2,17 +2,17 @@
 //
 // One workgroup owns BM = NW*QT*32 consecutive query rows of one (sequence, head) pair and walks
 // the key/value rows of that sequence in tiles of BN.  All matrix work is on
-// v_mfma_f32_32x32x16_{bf16,f16}, computed transposed so that no register shuffle is needed
+// v_mfma_f32_32x32x16_{bf16,f16,fp8_fp8}, computed transposed so that no register shuffle is needed
 // between the two products:
 //
 //   S^T[kv, q] = K[kv, :] . Q[q, :]^T        A = K tile (LDS),   B = Q (registers, loaded once)
-//   P^T        = silu-part(S^T), masked      in registers, packed to 16 bit
+//   P^T        = silu-part(S^T), masked      in registers, packed to the operand type
 //   O^T[dv, q] += V^T[dv, kv] . P^T[kv, q]   A = V tile (LDS, transposing read), B = P^T (registers)
 //
 // The accumulator layout of a 32x32 MFMA holds, per lane, one column (a query row) and sixteen
 // rows (kv positions); taken eight at a time those sixteen values are exactly the B operand of
 // the second product, provided the A operand (V^T) enumerates the kv rows in the same order,
-// which the ds_read_b64_tr_b16 addressing below arranges.
+// which the ds_read_b64_tr_b16 / ds_read_b64_tr_b8 addressing below arranges.
 //
 // silu(alpha*s)/N is evaluated as  s * rcp(1 + exp2(-alpha*log2(e)*s))  per element and the
 // common factor alpha/N is applied once to the fp32 output.  There is no row max / row sum:
@@ -66,18 +66,78 @@ struct FwdParams {
     float oscale;       // (alpha / max_seq_len) / c1 = -1 / (max_seq_len * log2(e)); 0 if alpha == 0
 };
 
+// Element types.  ES = bytes per element; `vec8` = eight elements = one MFMA operand of a lane;
+// `out_elem` = type of the output tensor; PRESCALE_Q: multiply Q by c1 when it is loaded (otherwise c1 is
+// applied to the accumulator); `silu` maps one accumulator value to the P value that is rounded and
+// packed by `pack8`, leaving a constant factor to the output scale.
 struct Bf16 {
     typedef bf16x8_t vec8;
     typedef __bf16 elem;
+    typedef __bf16 out_elem;
+    static constexpr int ES = 2;
+    static constexpr bool PRESCALE_Q = true;
     static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    // accumulator already holds t = c1*s; p = t * sigmoid(alpha s) = t / (1 + 2^t)
+    static __device__ __forceinline__ float silu(float t, float) {
+        return t * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
+    }
+    static __device__ __forceinline__ vec8 pack8(const float (&p)[8]) {
+        vec8 r;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = (elem)p[j];
+        return r;
     }
 };
 struct Fp16 {
     typedef f16x8_t vec8;
     typedef _Float16 elem;
+    typedef _Float16 out_elem;
+    static constexpr int ES = 2;
+    static constexpr bool PRESCALE_Q = true;
     static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float silu(float t, float) {
+        return t * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
+    }
+    static __device__ __forceinline__ vec8 pack8(const float (&p)[8]) {
+        vec8 r;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r[j] = (elem)p[j];
+        return r;
+    }
+};
+// OCP e4m3 (torch.float8_e4m3fn) inputs with per-tensor scales, bf16 output.  Both products run on
+// v_mfma_f32_32x32x16_fp8_fp8.  Q cannot be pre-scaled in 8 bits, so c1 (which here also carries
+// q_scale*k_scale) multiplies the accumulator.  P is kept in e4m3 as 16 * t * sigmoid: the factor 16 puts
+// typical magnitudes (|t| around 1e-2) into the normal range of e4m3 (2^-6 .. 448); p is unbounded only
+// towards -inf (t -> -inf), where it is clamped to the largest finite e4m3 value.
+struct Fp8 {
+    typedef long vec8;
+    typedef unsigned char elem;
+    typedef __bf16 out_elem;
+    static constexpr int ES = 1;
+    static constexpr bool PRESCALE_Q = false;
+    static constexpr float PSCALE = 16.0f;
+    static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float silu(float raw, float c1) {
+        const float t = raw * c1;
+        const float e = __builtin_amdgcn_exp2f(t);
+        const float d = __builtin_fmaf(e, 1.0f / PSCALE, 1.0f / PSCALE);  // (1 + 2^t) / 16
+        const float p = t * __builtin_amdgcn_rcpf(d);
+        return __builtin_fmaxf(p, -448.0f);
+    }
+    static __device__ __forceinline__ vec8 pack8(const float (&p)[8]) {
+        int lo = 0, hi = 0;
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], lo, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], lo, true);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(p[4], p[5], hi, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(p[6], p[7], hi, true);
+        return (long)(((unsigned long)(unsigned)hi << 32) | (unsigned)lo);
     }
 };
 
@@ -116,15 +176,22 @@ struct SeqMask {
 // send those 16 rows to 16 different 16-byte slots of the 256-byte bank line.
 template <int CH>
 __device__ __forceinline__ int swz_k(int row) {
-    static_assert(CH == 4 || CH == 8 || CH == 16, "row of 64, 128 or 256 bytes");
+    static_assert(CH == 2 || CH == 4 || CH == 8 || CH == 16, "row of 32 .. 256 bytes");
     return (row / (16 / CH)) & (CH - 1);
 }
-// V tile, read with ds_read_b64_tr_b16: one instruction touches 8 rows (4 per half-wave) x one 64-byte
-// segment, 8 bytes per lane.  f must send rows r..r+3 to four different 64-byte bank groups and rows
-// r, r+4 to different 32-byte halves of a group.
-template <int CH>
+// V tile of 16-bit elements, read with ds_read_b64_tr_b16: one instruction touches 8 rows (4 per
+// half-wave) x one 64-byte segment, 8 bytes per lane.  f must send rows r..r+3 to four different 64-byte
+// bank groups and rows r, r+4 to different 32-byte halves of a group.
+// V tile of 8-bit elements (128-byte rows), read with ds_read_b64_tr_b8: a half-wave touches rows
+// {0..3, 8..11} + 4g, 32 bytes each (two 16-byte chunks 2dt, 2dt+1); rows of equal parity share a
+// 128-byte half of the bank line, so f spreads rows {0,2,8,10} (and {1,3,9,11}) over chunk pairs.
+template <int CH, int ES>
 __device__ __forceinline__ int swz_v(int row) {
-    static_assert(CH == 4 || CH == 8 || CH == 16, "row of 64, 128 or 256 bytes");
+    static_assert(CH == 2 || CH == 4 || CH == 8 || CH == 16, "row of 32 .. 256 bytes");
+    if (ES == 1) {
+        if (CH == 8) return (((row >> 1) & 1) | (((row >> 3) & 1) << 1)) << 1;
+        return 0;
+    }
     const int half_swap = ((row >> 2) & 1) << 1;
     if (CH == 16) return ((row & 3) << 2) | half_swap;
     if (CH == 8) return (((row >> 1) & 1) << 2) | half_swap;
@@ -250,27 +317,26 @@ struct RowMask {
     }
 };
 
-// P^T for one 32x32 block.  The accumulator holds t = c1*s with c1 = -alpha*log2(e) (Q was pre-scaled), so
-// s*sigmoid(alpha s) = (t / c1) * rcp(1 + exp2(t)); the kernel forms p = t * rcp(1 + exp2(t)) and leaves the
-// constant 1/c1 to the output scale.  p is zeroed where the mask says so, rounded to the 16-bit type and
-// packed as two MFMA B operands.
+// P^T for one 32x32 block.  With t = c1*s, c1 = -alpha*log2(e) (for 16-bit inputs the accumulator already
+// holds t because Q was pre-scaled), s*sigmoid(alpha s) = (t / c1) * rcp(1 + exp2(t)); the kernel forms
+// p = t * rcp(1 + exp2(t)) (TT::silu) and leaves the constant 1/c1 to the output scale.  p is zeroed where
+// the mask says so, rounded to the operand type and packed as two MFMA B operands.
 // `sp0` is the sequence position of this lane's first kv slot of the block.
 template <class TT, bool MASKED>
-__device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], const SeqMask& M,
+__device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], float c1, const SeqMask& M,
                                           const RowMask& row, int sp0) {
-    typedef typename TT::elem elem;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         // eight elements at a time, fenced, so that the scheduler cannot pile up temporaries of all sixteen
+        float p[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int r = half * 8 + j;
-            float x = s[r];
-            float e = __builtin_amdgcn_exp2f(x);
-            float pr = x * __builtin_amdgcn_rcpf(1.0f + e);
+            float pr = TT::silu(s[r], c1);
             if (MASKED) pr = row.valid(M, sp0 + 8 * (r >> 2) + (r & 3)) ? pr : 0.f;
-            pb[half][j] = (elem)pr;
+            p[j] = pr;
         }
+        pb[half] = TT::pack8(p);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
@@ -285,14 +351,17 @@ template <class TT, int KS>
 __device__ __forceinline__ void load_q_operand(typename TT::vec8 (&qreg)[KS], const char* q, int64_t qrow0, int ql, int nq,
                                                int64_t q_rs, int64_t q_hs, int h, int g, float qscale) {
     typedef typename TT::vec8 vec8;
-    typedef typename TT::elem elem;
+    constexpr int ES = TT::ES;
     ql = ql < nq ? ql : nq - 1;
-    const char* qp = q + ((qrow0 + ql) * q_rs + (int64_t)h * q_hs) * 2 + g * 16;
+    const char* qp = q + ((qrow0 + ql) * q_rs + (int64_t)h * q_hs) * ES + g * 8 * ES;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-        vec8 raw = *(const vec8*)(qp + ks * 32);
+        vec8 raw = *(const vec8*)(qp + ks * 16 * ES);
+        if constexpr (TT::PRESCALE_Q) {
+            typedef typename TT::elem elem;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) raw[j] = (elem)((float)raw[j] * qscale);
+            for (int j = 0; j < 8; ++j) raw[j] = (elem)((float)raw[j] * qscale);
+        }
         qreg[ks] = raw;
     }
 }
@@ -304,32 +373,56 @@ __device__ __forceinline__ void load_q_operand(typename TT::vec8 (&qreg)[KS], co
 // kv rows of dv i.  Operand lane l must end up with dv = l%32 and kv slots {4g..4g+3} (first read) and
 // {8+4g..8+4g+3} (second read), g = l/32 -- the order in which the accumulator of the first product
 // holds its kv rows.
-template <int DQK, int DV>
+template <class TT, int DQK, int DV>
 __device__ __forceinline__ void lds_read_offsets(int (&kaddr)[DQK / 16], int (&vaddr)[2][DV / 32], int lane) {
-    constexpr int KS = DQK / 16, DT = DV / 32, KROW = DQK * 2, VROW = DV * 2, KCH = DQK / 8, VCH = DV / 8;
+    constexpr int ES = TT::ES;
+    constexpr int KS = DQK / 16, DT = DV / 32, KROW = DQK * ES, VROW = DV * ES, KCH = KROW / 16, VCH = VROW / 16;
     const int g = lane >> 5, l32 = lane & 31;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) kaddr[ks] = l32 * KROW + (((2 * ks + g) ^ swz_k<KCH>(l32)) * 16);
+    for (int ks = 0; ks < KS; ++ks) {
+        const int byte = (16 * ks + 8 * g) * ES;  // eight consecutive elements of the row
+        kaddr[ks] = l32 * KROW + (((byte >> 4) ^ swz_k<KCH>(l32)) * 16) + (byte & 15);
+    }
     const int i16 = lane & 15, half = (lane >> 4) & 1;
-    const int jrow = i16 >> 2, q4 = i16 & 3;
+    if constexpr (ES == 2) {
+        const int jrow = i16 >> 2, q4 = i16 & 3;
 #pragma unroll
-    for (int sec = 0; sec < 2; ++sec) {
-        const int row = 8 * sec + 4 * g + jrow;  // + 32 sub + 16 t
+        for (int sec = 0; sec < 2; ++sec) {
+            const int row = 8 * sec + 4 * g + jrow;  // + 32 sub + 16 t
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const int chunk = dt * 4 + 2 * half + (q4 >> 1);
+                vaddr[sec][dt] = row * VROW + ((chunk ^ swz_v<VCH, ES>(row)) * 16) + (q4 & 1) * 8;
+            }
+        }
+    } else {
+        // ds_read_b64_tr_b8: within 16 lanes, lanes 2j and 2j+1 supply the address of 16 consecutive dv of
+        // kv row j (8 bytes each) and the hardware hands lane i the eight kv rows of dv i: one read fills
+        // all eight kv slots {4g..4g+3, 8+4g..8+4g+3} of the operand.
+        const int jrow = i16 >> 1, e = i16 & 1;
+        const int row = 8 * (jrow >> 2) + 4 * g + (jrow & 3);  // + 32 sub + 16 t
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const int chunk = dt * 4 + 2 * half + (q4 >> 1);
-            vaddr[sec][dt] = row * VROW + ((chunk ^ swz_v<VCH>(row)) * 16) + (q4 & 1) * 8;
+            const int chunk = dt * 2 + half;
+            vaddr[0][dt] = row * VROW + ((chunk ^ swz_v<VCH, ES>(row)) * 16) + e * 8;
+            vaddr[1][dt] = 0;
         }
     }
 }
 
-// A operand of the second product (32 dv x 16 kv) from two transposing LDS reads.
+// A operand of the second product (32 dv x 16 kv): two transposing LDS reads of four 16-bit elements, or
+// one of eight 8-bit elements.
 template <class TT>
 __device__ __forceinline__ typename TT::vec8 read_vt_operand(const char* lo_addr, const char* hi_addr) {
-    s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, lo_addr));
-    s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, hi_addr));
-    s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(typename TT::vec8, both);
+    if constexpr (TT::ES == 2) {
+        s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, lo_addr));
+        s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, hi_addr));
+        s16x8_t both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(typename TT::vec8, both);
+    } else {
+        i32x2_t v = __builtin_amdgcn_ds_read_tr8_b64_v2i32(HSTU_LDS(i32x2_t, lo_addr));
+        return __builtin_bit_cast(typename TT::vec8, v);
+    }
 }
 
 // out[q, dv] = oscale * O^T[dv, q] for one block of 32 query rows; the lane holds 4 consecutive dv per
@@ -337,7 +430,7 @@ __device__ __forceinline__ typename TT::vec8 read_vt_operand(const char* lo_addr
 template <class TT, int DT, int QT>
 __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int qt, char* o, int64_t orow0, int ql, int nq,
                                              int64_t o_rs, int64_t o_hs, int h, int g, float oscale) {
-    typedef typename TT::elem elem;
+    typedef typename TT::out_elem elem;  // 16 bits
     typedef __attribute__((ext_vector_type(4))) elem elem4;
     if (ql >= nq) return;
     char* op = o + ((orow0 + ql) * o_rs + (int64_t)h * o_hs) * 2 + g * 8;
@@ -365,20 +458,20 @@ __device__ __forceinline__ void global_load_lds16_soff(const char* base_uniform,
 
 // Copy `ROWS` rows of `ROWBYTES` bytes from global memory into LDS with the chunk swizzle.
 // Rows at or beyond `n_rows_valid` re-read the last valid row (their products are masked).
-template <int ROWS, int ROWBYTES, int NTHREADS, bool IS_V>
+template <int ROWS, int ROWBYTES, int NTHREADS, bool IS_V, int ES>
 __device__ __forceinline__ void load_tile_to_lds(const char* gbase, int64_t row_stride_bytes, int row0,
                                                  int last_row, char* lds_tile, int wave, int lane) {
     constexpr int CH = ROWBYTES / 16;                // 16-byte chunks per row
     constexpr int INSTR = ROWS * CH / 64;            // wave-wide copies per tile
     constexpr int NWAVES = NTHREADS / 64;
-    static_assert(INSTR % NWAVES == 0, "tile copy must split evenly over the waves");
 #pragma unroll
-    for (int i = 0; i < INSTR / NWAVES; ++i) {
+    for (int i = 0; i < (INSTR + NWAVES - 1) / NWAVES; ++i) {
         int inst = wave + i * NWAVES;
+        if (inst >= INSTR) break;  // narrow rows: fewer copies than waves
         int p = inst * 64 + lane;
         int row = p / CH;
         int phys = p % CH;
-        int logical = phys ^ (IS_V ? swz_v<CH>(row) : swz_k<CH>(row));
+        int logical = phys ^ (IS_V ? swz_v<CH, ES>(row) : swz_k<CH>(row));
         int grow = row0 + row;
         grow = grow > last_row ? last_row : grow;
         const char* src = gbase + (int64_t)grow * row_stride_bytes + logical * 16;

@@ -12,10 +12,10 @@ namespace hstu {
 template <class TT, int DQK, int DV, int QT, int BN, bool MASKED>
 __device__ __forceinline__ void tile_compute(const char* kt, const char* vt, const typename TT::vec8 (&qreg)[QT][DQK / 16],
                                              f32x16_t (&oacc)[DV / 32][QT], const int (&kaddr)[DQK / 16],
-                                             const int (&vaddr)[2][DV / 32], const SeqMask& M, int sp0,
+                                             const int (&vaddr)[2][DV / 32], float c1, const SeqMask& M, int sp0,
                                              const RowMask (&rows)[QT]) {
     typedef typename TT::vec8 vec8;
-    constexpr int NS = BN / 32, KS = DQK / 16, DT = DV / 32, KROW = DQK * 2, VROW = DV * 2;
+    constexpr int NS = BN / 32, KS = DQK / 16, DT = DV / 32, KROW = DQK * TT::ES, VROW = DV * TT::ES;
     // ---- S^T = K Q^T
     f32x16_t s[NS][QT];
 #pragma unroll
@@ -36,7 +36,7 @@ __device__ __forceinline__ void tile_compute(const char* kt, const char* vt, con
 #pragma unroll
     for (int sub = 0; sub < NS; ++sub)
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) silu_pack<TT, MASKED>(s[sub][qt], pb[sub][qt], M, rows[qt], sp0 + sub * 32);
+        for (int qt = 0; qt < QT; ++qt) silu_pack<TT, MASKED>(s[sub][qt], pb[sub][qt], c1, M, rows[qt], sp0 + sub * 32);
     // ---- O^T += V^T P^T
 #pragma unroll
     for (int sub = 0; sub < NS; ++sub)
@@ -57,7 +57,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     constexpr int BM = NW * QT * 32;
     constexpr int KS = DQK / 16;
     constexpr int DT = DV / 32;
-    constexpr int KROW = DQK * 2, VROW = DV * 2;
+    constexpr int ES = TT::ES;
+    constexpr int KROW = DQK * ES, VROW = DV * ES;
     constexpr int KTILE = BN * KROW, VTILE = BN * VROW, STAGE = KTILE + VTILE;
     constexpr int NT = NW * 64;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -80,13 +81,13 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     int jt = next_valid_tile<BN>(W, W.jt_begin);
     const int jt_end = W.jt_end;
 
-    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * 2;
-    const char* vbase = p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * 2;
-    const int64_t k_rsb = p.k_rs * 2, v_rsb = p.v_rs * 2;
+    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * ES;
+    const char* vbase = p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * ES;
+    const int64_t k_rsb = p.k_rs * ES, v_rsb = p.v_rs * ES;
 
     if (jt < jt_end) {
-        load_tile_to_lds<BN, KROW, NT, false>(kbase, k_rsb, jt * BN, n - 1, smem, wave, lane);
-        load_tile_to_lds<BN, VROW, NT, true>(vbase, v_rsb, jt * BN, n - 1, smem + KTILE, wave, lane);
+        load_tile_to_lds<BN, KROW, NT, false, ES>(kbase, k_rsb, jt * BN, n - 1, smem, wave, lane);
+        load_tile_to_lds<BN, VROW, NT, true, ES>(vbase, v_rsb, jt * BN, n - 1, smem + KTILE, wave, lane);
     }
 
     vec8 qreg[QT][KS];
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
 
     int kaddr[KS];
     int vaddr[2][DT];
-    lds_read_offsets<DQK, DV>(kaddr, vaddr, lane);
+    lds_read_offsets<TT, DQK, DV>(kaddr, vaddr, lane);
 
     f32x16_t oacc[DT][QT];
 #pragma unroll
@@ -118,16 +119,16 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
         __syncthreads();                      // ... for every wave, and the other stage is no longer read
         if (jn < jt_end) {
             char* nxt = smem + (stage ^ 1) * STAGE;
-            load_tile_to_lds<BN, KROW, NT, false>(kbase, k_rsb, jn * BN, n - 1, nxt, wave, lane);
-            load_tile_to_lds<BN, VROW, NT, true>(vbase, v_rsb, jn * BN, n - 1, nxt + KTILE, wave, lane);
+            load_tile_to_lds<BN, KROW, NT, false, ES>(kbase, k_rsb, jn * BN, n - 1, nxt, wave, lane);
+            load_tile_to_lds<BN, VROW, NT, true, ES>(vbase, v_rsb, jn * BN, n - 1, nxt + KTILE, wave, lane);
         }
 
         const int cls = M.classify(wR0, wR1, jt * BN, BN);
         const char* kt = smem + stage * STAGE;
         if (cls == 2) {
-            tile_compute<TT, DQK, DV, QT, BN, false>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, M, jt * BN + 4 * g, rows);
+            tile_compute<TT, DQK, DV, QT, BN, false>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
         } else if (cls == 1) {
-            tile_compute<TT, DQK, DV, QT, BN, true>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, M, jt * BN + 4 * g, rows);
+            tile_compute<TT, DQK, DV, QT, BN, true>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
         }
         jt = jn;
         stage ^= 1;

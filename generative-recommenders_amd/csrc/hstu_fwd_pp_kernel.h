@@ -27,7 +27,7 @@ namespace hstu {
 // Direct HBM -> LDS copy of one tile, spread over the four "A" waves (copies issued from the "B" waves'
 // matrix phase were measured to stall it; from the A waves they are free); per-lane byte offsets from the
 // tile's first row are precomputed.
-template <int ROWS, int ROWBYTES, bool IS_V>
+template <int ROWS, int ROWBYTES, bool IS_V, int ES>
 struct TileCopy {
     static constexpr int CH = ROWBYTES / 16;
     static constexpr int NI = ROWS * CH / 64;       // wave-wide copy instructions per tile
@@ -39,7 +39,7 @@ struct TileCopy {
         const int p = inst * 64 + lane;
         int row = p / CH;
         const int phys = p % CH;
-        const int logical = phys ^ (IS_V ? swz_v<CH>(row) : swz_k<CH>(row));
+        const int logical = phys ^ (IS_V ? swz_v<CH, ES>(row) : swz_k<CH>(row));
         row = row < max_row ? row : max_row;
         return (unsigned)(row * row_stride_bytes) + logical * 16;
     }
@@ -77,7 +77,8 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     constexpr int NS = BN / 32;
     constexpr int KS = DQK / 16;
     constexpr int DT = DV / 32;
-    constexpr int KROW = DQK * 2, VROW = DV * 2;
+    constexpr int ES = TT::ES;
+    constexpr int KROW = DQK * ES, VROW = DV * ES;
     constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
     constexpr int NSLOT = 3;
     // LDS: 3 K slots, then 3 V slots.  A static array (the only LDS object, so it sits at address 0) lets
@@ -126,11 +127,11 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     if (T <= 0) return;  // cannot happen for a row block with rows (each row sees itself); kept for safety
     int t_cur = W.jt_begin;
 
-    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * 2;
-    const char* vbase = p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * 2;
-    const int64_t k_rsb = p.k_rs * 2, v_rsb = p.v_rs * 2;
-    typedef TileCopy<BN, KROW, false> KCopy;
-    typedef TileCopy<BN, VROW, true> VCopy;
+    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * ES;
+    const char* vbase = p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * ES;
+    const int64_t k_rsb = p.k_rs * ES, v_rsb = p.v_rs * ES;
+    typedef TileCopy<BN, KROW, false, ES> KCopy;
+    typedef TileCopy<BN, VROW, true, ES> VCopy;
     KCopy kcopy;
     VCopy vcopy;
     kcopy.init(wave, lane, k_rsb, n);
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
 
     int kaddr[KS];
     int vaddr[2][DT];
-    lds_read_offsets<DQK, DV>(kaddr, vaddr, lane);
+    lds_read_offsets<TT, DQK, DV>(kaddr, vaddr, lane);
 #pragma unroll
     for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
@@ -263,10 +264,10 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     auto valu_phase = [&](int tile) __attribute__((always_inline)) {
         if (tile >= full_begin && tile < full_end) {
 #pragma unroll
-            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, false>(s[sub], pb[sub], M, row, 0);
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, false>(s[sub], pb[sub], p.c1, M, row, 0);
         } else {
 #pragma unroll
-            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, true>(s[sub], pb[sub], M, row, tile * BN + 4 * g + sub * 32);
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, true>(s[sub], pb[sub], p.c1, M, row, tile * BN + 4 * g + sub * 32);
         }
     };
     auto end_of_step = [&]() __attribute__((always_inline)) {

@@ -316,3 +316,71 @@ def test_wrapper_rejects_what_it_cannot_do(pkg, dev):
     with torch.no_grad():
         pkg.hstu_mha(32, 0.1, qg, k.to(dev), v.to(dev), offs.to(dev))
     torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------- fp8 (e4m3, per-tensor scales, bf16 out)
+def _quantize(x):
+    """Per-tensor scale from absmax, as the baseline configuration states: x ~ x_q * scale."""
+    scale = float(x.float().abs().max()) / 448.0
+    xq = (x.float() / scale).to(torch.float8_e4m3fn)
+    return xq, scale
+
+
+def _cos(a, b):
+    a, b = a.float().flatten().double(), b.float().flatten().double()
+    return float((a @ b) / (a.norm() * b.norm()))
+
+
+FP8_CASES = [
+    # name, lengths, targets, N, w, c, D, H
+    ("causal_d128", [700, 64, 1, 333, 0, 1200], None, 1200, 0, 0, 128, 2),
+    ("targets_d128", [900, 300, 2100], [64, 200, 256], 2100, 0, 0, 128, 4),
+    ("window_ctx_targets_d128", [1500, 260, 77], [100, 130, 5], 1536, 300, 6, 128, 2),
+    ("d64", [500, 129], [20, 3], 512, 0, 0, 64, 2),
+    ("d32", [300, 64], None, 320, 40, 0, 32, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("e", FP8_CASES, ids=[e[0] for e in FP8_CASES])
+def test_fp8_against_oracle(pkg, dev, e, cfg):
+    """cosine >= 0.995 against the oracle on the un-quantised inputs (the stated bar for fp8), and a tighter
+    bound against the oracle fed the de-quantised inputs, which isolates the kernel from input quantisation."""
+    name, lengths, targets, N, w, c, D, H = e
+    _announce("fp8", name, "cfg", cfg)
+    q, k, v, offs, t = make_case(91, lengths, H, D, targets=targets, dtype=torch.float32)
+    (qq, qs), (kq, ks), (vq, vs) = _quantize(q), _quantize(k), _quantize(v)
+    alpha = 1.0 / D**0.5
+    got = pkg.hstu_mha(
+        N, alpha, qq.to(dev), kq.to(dev), vq.to(dev), offs.to(dev), num_targets=None if t is None else t.to(dev),
+        max_attn_len=w, contextual_seq_len=c, q_scale=qs, k_scale=ks, v_scale=vs, tile_config=cfg,
+    )
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and got.shape == v.shape
+    assert torch.isfinite(got.float()).all()
+    ref = _ref_full(q, k, v, offs, t, N, alpha, w, c)
+    ref_q = _ref_full(qq.float() * qs, kq.float() * ks, vq.float() * vs, offs, t, N, alpha, w, c)
+    cos, cos_q = _cos(got.cpu(), ref), _cos(got.cpu(), ref_q)
+    assert cos >= 0.995, f"{name}: cosine vs un-quantised oracle {cos:.5f}"
+    assert cos_q >= 0.998, f"{name}: cosine vs de-quantised oracle {cos_q:.5f}"
+    rel = float((got.float().cpu() - ref_q).norm() / ref_q.norm())
+    assert rel <= 0.06, f"{name}: relative error vs de-quantised oracle {rel:.4f}"
+
+
+def test_fp8_delta_and_scales(pkg, dev):
+    """Delta form in fp8, and the scales really are applied: halving v_scale halves the output exactly."""
+    _announce("fp8 delta")
+    delta, D = 64, 128
+    lengths = [500 + delta, 90 + delta, delta]
+    q, k, v, offs, t = make_case(92, lengths, 2, D, targets=[delta] * 3, dtype=torch.float32)
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(3)])
+    dq = q[idx].contiguous()
+    (qq, qs), (kq, ks), (vq, vs) = _quantize(dq), _quantize(k), _quantize(v)
+    alpha = 1.0 / D**0.5
+    kw = dict(num_targets=t.to(dev), q_scale=qs, k_scale=ks)
+    got = pkg.delta_hstu_mha(700, alpha, qq.to(dev), kq.to(dev), vq.to(dev), offs.to(dev), v_scale=vs, **kw)
+    half = pkg.delta_hstu_mha(700, alpha, qq.to(dev), kq.to(dev), vq.to(dev), offs.to(dev), v_scale=vs / 2, **kw)
+    torch.cuda.synchronize()
+    ref = O.cached_hstu_mha_per_sequence(700, alpha, dq, k, v, offs, t)
+    assert _cos(got.cpu(), ref) >= 0.995
+    assert torch.equal(got.float(), half.float() * 2.0)
