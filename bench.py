@@ -22,6 +22,9 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
 PEAK_HBM_GBS = 8000.0
 HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced against HBM bandwidth
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
+# counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
+MEASURED_TRAFFIC_BYTES = {"headline": 2.742e9}
 
 
 def run_gpu(wl, args, pkg, workloads, torch):
@@ -65,27 +68,30 @@ def run_gpu(wl, args, pkg, workloads, torch):
 
 def run_cpu_baseline(wl, torch, workloads, budget_s=20.0):
     """The PyTorch oracle (per-sequence form of the reference's pytorch_hstu_mha, fp32) on a bounded sample."""
+    import numpy as np
+
     from oracle import hstu_oracle
 
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
-    inp = workloads.make_inputs(wl, torch.device("cpu"), dtype=torch.float32)
     order = sorted(range(wl.batch), key=lambda b: -int(wl.lengths[b]))
     # sample: the longest sequence first, then every 8th by length, until the time budget is spent
     picks = [order[0]] + order[8::8]
+    picks += [b for b in order if b not in picks]
     done, flops, t_used = [], 0.0, 0.0
     for b in picks:
         sub = workloads.Workload(
-            "s", 1, wl.heads, wl.dqk, wl.dv, wl.max_seq_len, wl.lengths[b : b + 1],
-            None if wl.num_targets is None else wl.num_targets[b : b + 1], wl.max_attn_len,
-            wl.contextual_seq_len, wl.min_full_attn_seq_len, wl.delta_size, wl.dtype, wl.alpha,
+            "s", 1, wl.heads, wl.dqk, wl.dv, wl.max_seq_len, np.asarray(wl.lengths[b : b + 1]),
+            None if wl.num_targets is None else np.asarray(wl.num_targets[b : b + 1]), wl.max_attn_len,
+            wl.contextual_seq_len, wl.min_full_attn_seq_len, wl.delta_size, wl.dtype, wl.alpha, wl.seed + b,
         )
+        inp = workloads.make_inputs(sub, torch.device("cpu"), dtype=torch.float32)
         t0 = time.perf_counter()
         hstu_oracle.hstu_mha_per_sequence(
             wl.max_seq_len, wl.alpha, inp["q"], inp["k"], inp["v"], inp["seq_offsets"], num_targets=inp["num_targets"],
             max_attn_len=wl.max_attn_len, contextual_seq_len=wl.contextual_seq_len,
-            min_full_attn_seq_len=wl.min_full_attn_seq_len, delta_size=wl.delta_size, sequences=[b],
+            min_full_attn_seq_len=wl.min_full_attn_seq_len, delta_size=wl.delta_size,
         )
         t_used += time.perf_counter() - t0
         flops += workloads.algorithmic_flops(sub)
@@ -111,6 +117,8 @@ def main():
     ap.add_argument("--tile-config", type=int, default=0)
     ap.add_argument("--fused-buffer", action="store_true", help="q/k/v as column slices of one [L,H,3D] buffer")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain 1 GiB device copy, so that a counter run can scale FETCH_SIZE/WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
@@ -128,6 +136,13 @@ def main():
     if wl.dtype == "fp32":
         print("bench.py: cfg1 is the CPU correctness case, not a GPU bench workload", file=sys.stderr)
         sys.exit(2)
+    if args.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     wall_ms, ev_ms = run_gpu(wl, args, pkg, workloads, torch)
     flops = workloads.algorithmic_flops(wl)
     ref_flops = workloads.reference_convention_flops(wl)
@@ -136,12 +151,12 @@ def main():
     if wl.name in HBM_BOUND:
         ach = nbytes / (ev_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None}
+                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
     else:
         peak = PEAK_TFLOPS[wl.dtype]
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(tflops / peak, 4), "traffic": None}
-    roof["kernel"] = "hstu_fwd_kernel"
+                "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
+    roof["kernel"] = "hstu_fwd_pp_kernel" if (args.tile_config == 2 or (args.tile_config == 0 and wl.max_seq_len >= 2048)) else "hstu_fwd_kernel"
     roof["kernel_ms"] = round(ev_ms, 4)
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = nbytes

@@ -285,7 +285,9 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     if (grp == 0) {
         // ---- A: [matrix(i) | VALU(i)] per step
         auto stepA = [&](auto slot_c) __attribute__((always_inline)) {
+            __builtin_amdgcn_s_setprio(3);  // the matrix core must not wait behind the other wave's VALU work
             matrix_phase(slot_c);
+            __builtin_amdgcn_s_setprio(0);
             __syncthreads();
             valu_phase(t_cur);
             end_of_step();
@@ -312,7 +314,9 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
         auto stepB = [&](auto slot_c) __attribute__((always_inline)) {
             valu_phase(t_cur - 1);
             __syncthreads();
+            __builtin_amdgcn_s_setprio(3);
             matrix_phase(slot_c);
+            __builtin_amdgcn_s_setprio(0);
             end_of_step();
             ++t_cur;
         };
