@@ -33,6 +33,7 @@ def run_gpu(wl, args, pkg, workloads, torch):
     q, k, v = inp["q"], inp["k"], inp["v"]
     kw = dict(num_targets=inp["num_targets"], max_attn_len=wl.max_attn_len, contextual_seq_len=wl.contextual_seq_len,
               tile_config=args.tile_config)
+    sort_kw = dict(sort_by_length=not args.no_sort)  # the reference's bench sets the same hint for its native path
     scales = {}
     if wl.dtype == "fp8":
         qs, ks, vs = [float(x.float().abs().max()) / 448.0 for x in (q, k, v)]
@@ -46,7 +47,7 @@ def run_gpu(wl, args, pkg, workloads, torch):
     else:
         def step():
             return pkg.hstu_mha(wl.max_seq_len, wl.alpha, q, k, v, inp["seq_offsets"],
-                                min_full_attn_seq_len=wl.min_full_attn_seq_len, **kw, **scales)
+                                min_full_attn_seq_len=wl.min_full_attn_seq_len, **kw, **scales, **sort_kw)
 
     for _ in range(args.warmup):
         out = step()
@@ -117,6 +118,7 @@ def main():
     ap.add_argument("--tile-config", type=int, default=0)
     ap.add_argument("--fused-buffer", action="store_true", help="q/k/v as column slices of one [L,H,3D] buffer")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sort", action="store_true", help="do not pass sort_by_length=True to hstu_mha")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 1 GiB device copy, so that a counter run can scale FETCH_SIZE/WRITE_SIZE")
     args = ap.parse_args()

@@ -10,7 +10,31 @@
 #include "hstu_fwd_kernel.h"
 #include "hstu_fwd_pp_kernel.h"
 
+namespace hstu {
+
+// order[rank] = sequence index, longest sequence first (ties by index).  One thread per sequence, each
+// counting the sequences that precede it; the offsets array is small and stays in cache.
+__global__ __launch_bounds__(256) void hstu_rank_kernel(const void* offsets, int offsets_i64, int B, int* order) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= B) return;
+    auto len = [&](int j) -> long long {
+        return offsets_i64 ? ((const long long*)offsets)[j + 1] - ((const long long*)offsets)[j]
+                           : (long long)(((const int*)offsets)[j + 1] - ((const int*)offsets)[j]);
+    };
+    const long long ni = len(i);
+    int rank = 0;
+    for (int j = 0; j < B; ++j) {
+        const long long nj = len(j);
+        rank += (nj > ni) || (nj == ni && j < i);
+    }
+    order[rank] = i;
+}
+
+}  // namespace hstu
+
 namespace {
+
+constexpr int kMaxSortBatch = 8192;  // beyond this the quadratic ranking is not worth its time
 
 thread_local char g_last_error[256] = "";
 
@@ -30,7 +54,7 @@ const TileConfig kConfigs[] = {
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
 template <class TT, int DQK, int DV, int QT, int NW, int BN, int OCC>
-int launch(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
+int launch(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
     constexpr int BM = NW * QT * 32;
     constexpr int smem = 2 * BN * (DQK + DV) * TT::ES;
     auto kern = hstu::hstu_fwd_kernel<TT, DQK, DV, QT, NW, BN, OCC>;
@@ -45,9 +69,11 @@ int launch(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
     }
     (void)BM;
     const int pairs_per_xcd = (num_pairs + 7) / 8;
-    const long long grid = (long long)pairs_per_xcd * 8 * p.num_mb;
+    const long long grid = (long long)pairs_per_xcd * 8 * p0.num_mb;
     if (grid <= 0) return HSTU_OK;
     if (grid > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    hstu::FwdParams p = p0;
+    p.pairs_per_xcd = pairs_per_xcd;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), smem, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -58,13 +84,15 @@ int launch(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
 }
 
 template <class TT, int DQK, int DV, int BN>
-int launch_pp(const hstu::FwdParams& p, int num_pairs, hipStream_t stream) {
+int launch_pp(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
     constexpr int smem = 0;  // the kernel's LDS is a static array
     auto kern = hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN>;
     const int pairs_per_xcd = (num_pairs + 7) / 8;
-    const long long grid = (long long)pairs_per_xcd * 8 * p.num_mb;
+    const long long grid = (long long)pairs_per_xcd * 8 * p0.num_mb;
     if (grid <= 0) return HSTU_OK;
     if (grid > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    hstu::FwdParams p = p0;
+    p.pairs_per_xcd = pairs_per_xcd;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -121,6 +149,11 @@ const char* hstu_hip_status_string(int status) {
 
 const char* hstu_hip_last_error(void) { return g_last_error; }
 
+size_t hstu_hip_workspace_bytes(const HstuFwdArgs* a) {
+    if (!a || !a->sort_by_length || a->batch < 2 || a->batch > kMaxSortBatch) return 0;
+    return (size_t)a->batch * sizeof(int);
+}
+
 int hstu_hip_tile_configs(void) { return kNumConfigs; }
 
 const char* hstu_hip_tile_config_name(int id) {
@@ -138,6 +171,7 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     if (a->delta_size == 0 && a->total_q != a->total_kv) return HSTU_ERR_BAD_SHAPE;
     if (a->total_kv > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     if (a->tile_config < 0 || a->tile_config > kNumConfigs) return HSTU_ERR_BAD_SHAPE;
+    if (a->workspace && (a->workspace_bytes < 0 || (reinterpret_cast<uintptr_t>(a->workspace) & 3) != 0)) return HSTU_ERR_MISALIGNED;
     if (a->dqk != a->dv) return HSTU_ERR_BAD_HEAD_DIM;  // as the reference's native op, flash_common.cpp:543-545
     if (a->dqk != 32 && a->dqk != 64 && a->dqk != 128) return HSTU_ERR_BAD_HEAD_DIM;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;  // nothing to do; pointers may be anything
@@ -191,6 +225,20 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
         // value scale and the factor P is stored with go into the output scale
         p.c1 *= a->q_scale * a->k_scale;
         p.oscale *= a->v_scale / hstu::Fp8::PSCALE;
+    }
+
+    // optional schedule: rank the sequences by length into the caller's scratch memory
+    const size_t ws_need = hstu_hip_workspace_bytes(a);
+    if (ws_need > 0 && a->workspace && (size_t)a->workspace_bytes >= ws_need) {
+        int* order = (int*)a->workspace;
+        hipLaunchKernelGGL(hstu::hstu_rank_kernel, dim3((a->batch + 255) / 256), dim3(256), 0, stream, a->seq_offsets,
+                           a->seq_offsets_i64, a->batch, order);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            set_last_error("rank kernel launch", e);
+            return HSTU_ERR_LAUNCH;
+        }
+        p.order = order;
     }
 
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;

@@ -58,7 +58,9 @@ struct FwdParams {
     const void* targets;
     int offsets_i64, targets_i64;
     int B, H;
+    const int* order;   // NULL, or sequence indices sorted by decreasing length (scheduling only)
     int num_mb;         // row blocks per (sequence, head) pair in the grid
+    int pairs_per_xcd;  // ceil(B*H / 8)
     int max_seq_len;
     int delta;          // 0 = full attention
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
@@ -234,14 +236,30 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
     const int bid = blockIdx.x;
     const int xcd = bid & 7;
     const int slot = bid >> 3;
-    const int pair = (slot / p.num_mb) * 8 + xcd;
+    // Heaviest work first.  Within a pair that is the last row block -- except that with a contextual prefix
+    // the first row block (its contextual rows see every non-target key) is the heaviest of all and runs
+    // many times longer than the others, so the first row blocks of all pairs are launched before anything else.
+    int pair_local, mb;
+    if (p.c > 0) {
+        if (slot < p.pairs_per_xcd) {
+            pair_local = slot;
+            mb = 0;
+        } else {
+            const int s2 = slot - p.pairs_per_xcd;
+            pair_local = s2 / (p.num_mb - 1);
+            mb = p.num_mb - 1 - (s2 - pair_local * (p.num_mb - 1));
+        }
+    } else {
+        pair_local = slot / p.num_mb;
+        mb = p.num_mb - 1 - (slot - pair_local * p.num_mb);
+    }
+    const int pair = pair_local * 8 + xcd;
     if (pair >= p.B * p.H) return false;
-    // heaviest row block first: the last one -- except that with a contextual prefix the first row block
-    // (its contextual rows see every non-target key) is the heaviest of all
-    const int rank = slot % p.num_mb;
-    const int mb = p.c > 0 ? (rank == 0 ? 0 : p.num_mb - rank) : p.num_mb - 1 - rank;
-    w.b = pair / p.H;
-    w.h = pair - w.b * p.H;
+    const int rseq = pair / p.H;
+    w.h = pair - rseq * p.H;
+    // `order` lists the sequences longest first, so that long sequences start early and are dealt evenly
+    // over the XCDs; it changes the schedule, never the result
+    w.b = p.order ? __builtin_amdgcn_readfirstlane(p.order[rseq]) : rseq;
     int64_t seq_start, seq_end;
     if (p.offsets_i64) {
         seq_start = ((const int64_t*)p.offsets)[w.b];

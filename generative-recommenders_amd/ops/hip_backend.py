@@ -48,7 +48,9 @@ class HstuFwdArgs(ctypes.Structure):
         ("k_scale", ctypes.c_float),
         ("v_scale", ctypes.c_float),
         ("tile_config", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("sort_by_length", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_int64),
     ]
 
 
@@ -58,6 +60,7 @@ EXPORTS = (
     "hstu_hip_last_error",
     "hstu_hip_check_args",
     "hstu_hip_mha_fwd",
+    "hstu_hip_workspace_bytes",
     "hstu_hip_tile_configs",
     "hstu_hip_tile_config_name",
 )
@@ -87,6 +90,8 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_check_args.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_mha_fwd.restype = ctypes.c_int
         L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
+        L.hstu_hip_workspace_bytes.restype = ctypes.c_size_t
+        L.hstu_hip_workspace_bytes.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_tile_configs.restype = ctypes.c_int
         L.hstu_hip_tile_config_name.restype = ctypes.c_char_p
         L.hstu_hip_tile_config_name.argtypes = [ctypes.c_int]
@@ -149,6 +154,7 @@ def mha_fwd(
     k_scale: float = 1.0,
     v_scale: float = 1.0,
     tile_config: int = 0,
+    sort_by_length: bool = False,
 ) -> None:
     """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors."""
     a = HstuFwdArgs()
@@ -179,6 +185,14 @@ def mha_fwd(
     a.dtype = _dtype_code(q.dtype)
     a.q_scale, a.k_scale, a.v_scale = q_scale, k_scale, v_scale
     a.tile_config = tile_config
+    a.sort_by_length = 1 if sort_by_length else 0
+    workspace = None
+    need = lib().hstu_hip_workspace_bytes(ctypes.byref(a))
+    if need > 0:
+        # scratch for the schedule; the caching allocator keeps it alive until the stream has consumed it
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+        a.workspace = workspace.data_ptr()
+        a.workspace_bytes = need
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         rc = lib().hstu_hip_mha_fwd(ctypes.byref(a), ctypes.c_void_p(stream))

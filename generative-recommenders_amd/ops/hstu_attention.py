@@ -4,7 +4,8 @@ Mirrors ``generative_recommenders/ops/hstu_attention.py`` of the reference (``hs
 at lines 101-207, ``delta_hstu_mha`` at lines 210-284): same argument names, defaults, assertion
 messages and output shapes.  Differences, all explicit:
 
-* there is one backend, so ``kernel`` / ``enable_tma`` / ``sort_by_length`` are accepted and ignored;
+* there is one backend, so ``kernel`` / ``enable_tma`` are accepted and ignored; ``sort_by_length`` is, as in
+  the reference, a scheduling hint (long sequences are started first) that never changes the result;
 * forward only -- inputs that require grad under ``torch.enable_grad()`` raise ``NotImplementedError``;
 * tensors must live on a HIP device; there is no CPU or PyTorch fallback;
 * fp8 (``torch.float8_e4m3fn``) q/k/v take per-tensor scales through ``q_scale``/``k_scale``/``v_scale``
@@ -120,6 +121,7 @@ def hstu_mha(
         k_scale=k_scale,
         v_scale=v_scale,
         tile_config=tile_config,
+        sort_by_length=sort_by_length,
     )
     return out
 

@@ -73,7 +73,12 @@ typedef struct HstuFwdArgs {
     int32_t dtype;                   /* HstuDtype */
     float q_scale, k_scale, v_scale; /* FP8 only: real value = stored value * scale (per tensor) */
     int32_t tile_config;             /* 0 = choose automatically; otherwise a value of hstu_hip_tile_configs() */
-    int32_t reserved;
+    int32_t sort_by_length;          /* scheduling hint of the reference (hstu_attention.py:115): start long
+                                        sequences first.  Needs `workspace`; never changes the result */
+    void* workspace;                 /* NULL, or device scratch of at least hstu_hip_workspace_bytes() bytes,
+                                        4-byte aligned, owned by the caller, free to reuse once the call's work on
+                                        `stream` has run */
+    int64_t workspace_bytes;
 } HstuFwdArgs;
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -97,6 +102,13 @@ int hstu_hip_check_args(const HstuFwdArgs* args);
  * delta-query (M-FALCON) forms.
  */
 int hstu_hip_mha_fwd(const HstuFwdArgs* args, void* stream);
+
+/*
+ * Bytes of `workspace` the call would use with these arguments (0 if it needs none).  The library never
+ * allocates: the reference's native op allocates its tile semaphore itself (flash_common.cpp:668-678);
+ * here the caller passes scratch memory, or NULL to run without the options that need it.
+ */
+size_t hstu_hip_workspace_bytes(const HstuFwdArgs* args);
 
 /* Number of selectable tile configurations and a short name for each (1-based ids). */
 int hstu_hip_tile_configs(void);

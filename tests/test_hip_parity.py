@@ -384,3 +384,27 @@ def test_fp8_delta_and_scales(pkg, dev):
     ref = O.cached_hstu_mha_per_sequence(700, alpha, dq, k, v, offs, t)
     assert _cos(got.cpu(), ref) >= 0.995
     assert torch.equal(got.float(), half.float() * 2.0)
+
+
+@pytest.mark.parametrize("cfg", [1, 2])
+def test_sort_by_length_changes_only_the_schedule(pkg, dev, cfg):
+    """`sort_by_length` (hstu_attention.py:115 of the reference) reorders the launch; the result is bit-identical."""
+    _announce("sort_by_length", cfg)
+    rng = np.random.default_rng(8)
+    lengths = rng.integers(0, 900, size=37)
+    lengths[5] = 2300
+    q, k, v, offs, t = make_case(55, lengths, 2, 128, targets=np.minimum(lengths, rng.integers(0, 40, size=37)))
+    args = (2304, 0.09, q.to(dev), k.to(dev), v.to(dev), offs.to(dev))
+    kw = dict(num_targets=t.to(dev), max_attn_len=500, contextual_seq_len=0, tile_config=cfg)
+    a = pkg.hstu_mha(*args, **kw)
+    b = pkg.hstu_mha(*args, sort_by_length=True, **kw)
+    kw["contextual_seq_len"] = 3
+    lengths_ok = torch.as_tensor(lengths) - t >= 3
+    if bool(lengths_ok.all()):
+        c1 = pkg.hstu_mha(*args, **kw)
+        c2 = pkg.hstu_mha(*args, sort_by_length=True, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(c1, c2)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert_parity(a, _ref_full(q, k, v, offs, t, 2304, 0.09, 500, 0), "sorted")
