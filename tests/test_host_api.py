@@ -86,6 +86,16 @@ def test_check_args_status_codes(backend):
     assert chk(delta_size=8, total_q=16) == 0
     assert chk(tile_config=99) == -5
     assert chk(total_q=0, total_kv=0, q=None) == 0  # empty input: nothing is dereferenced
+    # fp8 rows are 16-byte aligned at multiples of 16 elements; bf16 at multiples of 8
+    assert chk(dtype=2) == 0
+    assert chk(dtype=2, k_row_stride=4 * 128 + 8) == -4
+    assert chk(dtype=0, k_row_stride=4 * 128 + 8) == 0
+    assert chk(workspace=0x1002, workspace_bytes=64) == -4
+    # workspace is only asked for by sort_by_length, one int per sequence
+    need = lambda **o: backend.lib().hstu_hip_workspace_bytes(ctypes.byref(_args(backend, **o)))  # noqa: E731
+    assert need() == 0
+    assert need(sort_by_length=1, batch=64) == 256
+    assert need(sort_by_length=1, batch=1) == 0
     for rc in range(-8, 1):
         assert backend.lib().hstu_hip_status_string(rc)
     with pytest.raises(RuntimeError):
