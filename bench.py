@@ -158,7 +158,9 @@ def main():
         peak = PEAK_TFLOPS[wl.dtype]
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
-    roof["kernel"] = "hstu_fwd_pp_kernel" if (args.tile_config == 2 or (args.tile_config == 0 and wl.max_seq_len >= 2048)) else "hstu_fwd_kernel"
+    auto_cfg = 2 if (wl.delta_size == 0 and wl.total_kv // wl.batch >= 3072) else 3  # the library's own rule
+    cfg = args.tile_config or auto_cfg
+    roof["kernel"] = {1: "hstu_fwd_kernel", 2: "hstu_fwd_pp_kernel<NG=2>", 3: "hstu_fwd_pp_kernel<NG=1>"}[cfg]
     roof["kernel_ms"] = round(ev_ms, 4)
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = nbytes

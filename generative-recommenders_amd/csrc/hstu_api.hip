@@ -50,6 +50,7 @@ struct TileConfig {
 const TileConfig kConfigs[] = {
     {"m128n64w4", 1, 4, 64},
     {"m256n64w8pp", 1, 8, 64},
+    {"m128n64w4pl", 1, 4, 64},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -83,17 +84,17 @@ int launch(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
     return HSTU_OK;
 }
 
-template <class TT, int DQK, int DV, int BN>
+template <class TT, int DQK, int DV, int BN, int NG>
 int launch_pp(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
     constexpr int smem = 0;  // the kernel's LDS is a static array
-    auto kern = hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN>;
+    auto kern = hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN, NG>;
     const int pairs_per_xcd = (num_pairs + 7) / 8;
     const long long grid = (long long)pairs_per_xcd * 8 * p0.num_mb;
     if (grid <= 0) return HSTU_OK;
     if (grid > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     hstu::FwdParams p = p0;
     p.pairs_per_xcd = pairs_per_xcd;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), smem, stream, p);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NG * 256), smem, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_last_error("kernel launch", e);
@@ -107,7 +108,11 @@ int launch_cfg(const hstu::FwdParams& p0, int cfg, int rows_per_pair, int num_pa
     hstu::FwdParams p = p0;
     if (cfg == 2) {
         p.num_mb = (rows_per_pair + 255) / 256;
-        return launch_pp<TT, D, D, 64>(p, num_pairs, stream);
+        return launch_pp<TT, D, D, 64, 2>(p, num_pairs, stream);
+    }
+    if (cfg == 3) {
+        p.num_mb = (rows_per_pair + 127) / 128;
+        return launch_pp<TT, D, D, 64, 1>(p, num_pairs, stream);
     }
     p.num_mb = (rows_per_pair + 127) / 128;
     return launch<TT, D, D, 1, 4, 64, 2>(p, num_pairs, stream);
@@ -245,10 +250,11 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     const long long num_pairs_ll = (long long)a->batch * a->heads;
     if (num_pairs_ll > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     const int num_pairs = (int)num_pairs_ll;
-    // Automatic choice: the ping-pong kernel (256-row blocks, one workgroup per CU) wins once sequences
-    // are long enough to keep its pipeline full; short sequences waste less in 128-row blocks.
+    // Automatic choice, from sizes the host knows without reading the offsets: the ping-pong kernel (256-row
+    // blocks, one workgroup per CU) wins when the average sequence is long; the one-group pipeline (128-row
+    // blocks, two workgroups per CU) wastes less on short or very uneven sequences and in delta mode.
     int cfg = a->tile_config;
-    if (cfg == 0) cfg = a->max_seq_len >= 2048 ? 2 : 1;
+    if (cfg == 0) cfg = (a->delta_size == 0 && a->total_kv / a->batch >= 3072) ? 2 : 3;
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
     if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
     return launch_dim<hstu::Fp8>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);

@@ -69,19 +69,24 @@ struct TileCopy {
     }
 };
 
-template <class TT, int DQK, int DV, int BN>
-__global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) {
+// NG = 2: the ping-pong kernel described above (8 waves, 256 rows, 3 LDS slots, one workgroup per CU).
+// NG = 1: the same pipeline with a single group (4 waves, 128 rows, 2 LDS slots, two workgroups per CU and one
+//         barrier per tile); the overlap of matrix and VALU work then comes from the two workgroups that share a
+//         CU.  It wastes less on short sequences, whose last 256-row block would be mostly empty.
+template <class TT, int DQK, int DV, int BN, int NG>
+__global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParams p) {
     typedef typename TT::vec8 vec8;
     static_assert(DQK == DV, "the interleaved matrix phase assumes as many first-product as second-product MFMAs");
-    constexpr int BM = 256;
+    static_assert(NG == 1 || NG == 2, "one or two wave groups");
+    constexpr int BM = NG * 128;
     constexpr int NS = BN / 32;
     constexpr int KS = DQK / 16;
     constexpr int DT = DV / 32;
     constexpr int ES = TT::ES;
     constexpr int KROW = DQK * ES, VROW = DV * ES;
     constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
-    constexpr int NSLOT = 3;
-    // LDS: 3 K slots, then 3 V slots.  A static array (the only LDS object, so it sits at address 0) lets
+    constexpr int NSLOT = NG == 2 ? 3 : 2;
+    // LDS: NSLOT K slots, then NSLOT V slots.  A static array (the only LDS object, so it sits at address 0) lets
     // every tile and slot offset fold into the immediate field of the LDS reads.
     __shared__ __attribute__((aligned(1024))) char smem[NSLOT * (KTILE + VTILE)];
     constexpr int VOFF = NSLOT * KTILE;
@@ -94,7 +99,7 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int grp = wave >> 2;    // 0: waves 0-3 (A), 1: waves 4-7 (B); waves w and w+4 share a SIMD
+    const int grp = NG == 2 ? wave >> 2 : 0;  // 0: waves 0-3 (A), 1: waves 4-7 (B); waves w and w+4 share a SIMD
     const int g = lane >> 5;
     const int l32 = lane & 31;
 
@@ -139,11 +144,16 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     constexpr int NPW = KCopy::PER_WAVE + VCopy::PER_WAVE;  // copy instructions per wave and step
     static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
 
-    // before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1
+    // Copy schedule.  With 3 slots, step i copies V(i+1) and K(i+2) and its end waits for the copies of step
+    // i-1; before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1.  With 2 slots, step i copies
+    // V(i) and K(i+1) and waits for them at its own end; before step 0 only K(t0) is copied.
+    constexpr int AHEAD = NSLOT - 2;  // 1 or 0
     if (grp == 0) {
         kcopy.issue(kbase, k_rsb, t_cur * BN, n, smem, wave);
-        vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
-        kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
+        if (NSLOT == 3) {
+            vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
+            kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
+        }
     }
 
     vec8 qreg[KS];
@@ -182,12 +192,12 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     auto issue_copy = [&](auto slot_c, int j) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
         if (grp != 0) return;
-        const int tv = t_cur + 1 < jt_end ? t_cur + 1 : jt_end - 1;
-        const int tk = t_cur + 2 < jt_end ? t_cur + 2 : jt_end - 1;
+        const int tv = t_cur + AHEAD < jt_end ? t_cur + AHEAD : jt_end - 1;
+        const int tk = t_cur + AHEAD + 1 < jt_end ? t_cur + AHEAD + 1 : jt_end - 1;
         if (j < VCopy::PER_WAVE)
-            vcopy.issue_one(j, vbase, v_rsb, tv * BN, n, smem + VOFF + ((SLOT + 1) % NSLOT) * VTILE, wave);
+            vcopy.issue_one(j, vbase, v_rsb, tv * BN, n, smem + VOFF + ((SLOT + AHEAD) % NSLOT) * VTILE, wave);
         else
-            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, n, smem + ((SLOT + 2) % NSLOT) * KTILE, wave);
+            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, n, smem + ((SLOT + AHEAD + 1) % NSLOT) * KTILE, wave);
     };
     // S^T = K Q^T only (first step), K slot chosen at run time.
     auto gemm1_only = [&](int kslot) __attribute__((always_inline)) {
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
     auto matrix_phase = [&](auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
         const char* kt = smem + SLOT * KTILE;
-        const char* vt = smem + (VOFF - VBIAS) + ((SLOT + 2) % NSLOT) * VTILE;
+        const char* vt = smem + (VOFF - VBIAS) + ((SLOT + NSLOT - 1) % NSLOT) * VTILE;
         auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
             const int o = k >> 1;
             if ((k & 1) == 0) {
@@ -271,24 +281,26 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
         }
     };
     auto end_of_step = [&]() __attribute__((always_inline)) {
-        // every copy but this step's has landed for this wave ...
-        __builtin_amdgcn_s_waitcnt((NPW & 0xF) | ((NPW >> 4) << 14) | 0x0F70);
+        // 3 slots: every copy but this step's has landed for this wave; 2 slots: every copy ...
+        constexpr int LEAVE = NSLOT == 3 ? NPW : 0;
+        __builtin_amdgcn_s_waitcnt((LEAVE & 0xF) | ((LEAVE >> 4) << 14) | 0x0F70);
         __syncthreads();  // ... and for every wave
     };
     typedef std::integral_constant<int, 0> S0;
     typedef std::integral_constant<int, 1> S1;
     typedef std::integral_constant<int, 2> S2;
 
-    // Both groups execute the same barriers: two per step and one in the drain.  Step i uses slot i % 3;
-    // step 0 is peeled (first product only), then whole rounds of three steps, then the remainder.
-    const int rounds = (T - 1) / 3, rem = (T - 1) % 3;
+    // Both groups execute the same barriers: two per step and one in the drain (one group: one per step).
+    // Step i uses slot i % NSLOT; step 0 is peeled (first product only), then whole rounds of NSLOT steps,
+    // then the remainder.
+    const int rounds = (T - 1) / NSLOT, rem = (T - 1) % NSLOT;
     if (grp == 0) {
         // ---- A: [matrix(i) | VALU(i)] per step
         auto stepA = [&](auto slot_c) __attribute__((always_inline)) {
             __builtin_amdgcn_s_setprio(3);  // the matrix core must not wait behind the other wave's VALU work
             matrix_phase(slot_c);
             __builtin_amdgcn_s_setprio(0);
-            __syncthreads();
+            if (NG == 2) __syncthreads();
             valu_phase(t_cur);
             end_of_step();
             ++t_cur;
@@ -296,19 +308,27 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_pp_kernel(const FwdParams p) 
 #pragma unroll
         for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
         gemm1_only(0);
-        __syncthreads();
+        if (NG == 2) __syncthreads();
         valu_phase(t_cur);
         end_of_step();
         ++t_cur;
-        for (int r = 0; r < rounds; ++r) {
-            stepA(S1{});
-            stepA(S2{});
-            stepA(S0{});
+        if constexpr (NSLOT == 3) {
+            for (int r = 0; r < rounds; ++r) {
+                stepA(S1{});
+                stepA(S2{});
+                stepA(S0{});
+            }
+            if (rem >= 1) stepA(S1{});
+            if (rem >= 2) stepA(S2{});
+        } else {
+            for (int r = 0; r < rounds; ++r) {
+                stepA(S1{});
+                stepA(S0{});
+            }
+            if (rem >= 1) stepA(S1{});
         }
-        if (rem >= 1) stepA(S1{});
-        if (rem >= 2) stepA(S2{});
         gemm2_only((T - 1) % NSLOT);
-        __syncthreads();
+        if (NG == 2) __syncthreads();
     } else {
         // ---- B: [VALU(i-1) | matrix(i)] per step, one phase behind A
         auto stepB = [&](auto slot_c) __attribute__((always_inline)) {

@@ -49,7 +49,7 @@ def test_library_is_loaded_from_tree(pkg):
     assert os.path.dirname(hip_backend.library_path()).endswith(os.path.join("generative-recommenders_amd", "csrc"))
 
 
-@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("cfg", [1, 2, 3])
 def test_golden_fixture(pkg, dev, cfg):
     z = np.load(GOLDEN)
     for name in sorted({key.split(".")[0] for key in z.files}):
@@ -89,7 +89,7 @@ for _i in range(36):
             has_window=bool(_rng.integers(0, 2)),
             c=int(_rng.choice([0, 10])),
             dtype=[torch.bfloat16, torch.float16][int(_rng.integers(0, 2))],
-            cfg=int(_rng.choice([1, 2])),
+            cfg=int(_rng.choice([1, 2, 3])),
             i32=bool(_rng.integers(0, 2)),
         )
     )
@@ -142,7 +142,7 @@ EDGE = [
 ]
 
 
-@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("cfg", [1, 2, 3])
 @pytest.mark.parametrize("e", EDGE, ids=[e[0] for e in EDGE])
 def test_edge_cases(pkg, dev, e, cfg):
     name, lengths, targets, N, w, c, f = e
@@ -195,7 +195,7 @@ def test_inputs_not_modified_and_rows_all_written(pkg, dev):
     assert torch.isfinite(out.float()).all()
 
 
-@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("cfg", [1, 2, 3])
 @pytest.mark.parametrize("delta,w,c,D", [(8, 0, 0, 128), (256, 0, 0, 128), (130, 50, 4, 64), (1, 0, 0, 32), (20, 7, 0, 128)])
 def test_delta_against_oracle_and_tail_of_full(pkg, dev, delta, w, c, D, cfg):
     """delta_hstu_mha vs the oracle, and == the last rows of hstu_mha (hstu_attention_test.py:382-488)."""
@@ -341,7 +341,7 @@ FP8_CASES = [
 ]
 
 
-@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("cfg", [1, 2, 3])
 @pytest.mark.parametrize("e", FP8_CASES, ids=[e[0] for e in FP8_CASES])
 def test_fp8_against_oracle(pkg, dev, e, cfg):
     """cosine >= 0.995 against the oracle on the un-quantised inputs (the stated bar for fp8), and a tighter
@@ -386,7 +386,7 @@ def test_fp8_delta_and_scales(pkg, dev):
     assert torch.equal(got.float(), half.float() * 2.0)
 
 
-@pytest.mark.parametrize("cfg", [1, 2])
+@pytest.mark.parametrize("cfg", [1, 2, 3])
 def test_sort_by_length_changes_only_the_schedule(pkg, dev, cfg):
     """`sort_by_length` (hstu_attention.py:115 of the reference) reorders the launch; the result is bit-identical."""
     _announce("sort_by_length", cfg)
