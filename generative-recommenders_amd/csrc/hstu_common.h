@@ -41,6 +41,7 @@ typedef __attribute__((ext_vector_type(2))) int i32x2_t;
 
 #define HSTU_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
 #define HSTU_GLB(T, p) ((const __attribute__((address_space(1))) T*)(p))
+#define HSTU_CONST(T, p) ((const __attribute__((address_space(4))) T*)(p))
 
 __device__ __forceinline__ int64_t uniform64(int64_t x) {
     const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(uint64_t)x);
@@ -259,14 +260,17 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
     w.h = pair - rseq * p.H;
     // `order` lists the sequences longest first, so that long sequences start early and are dealt evenly
     // over the XCDs; it changes the schedule, never the result
-    w.b = p.order ? __builtin_amdgcn_readfirstlane(p.order[rseq]) : rseq;
+    // The index arrays are read-only for the whole launch and their addresses are wave-uniform: reading
+    // them through the constant address space makes these scalar loads (scalar cache, a fraction of the
+    // latency of a vector load), which matters because three of them are chained at the start of every workgroup.
+    w.b = p.order ? HSTU_CONST(int, p.order)[rseq] : rseq;
     int64_t seq_start, seq_end;
     if (p.offsets_i64) {
-        seq_start = ((const int64_t*)p.offsets)[w.b];
-        seq_end = ((const int64_t*)p.offsets)[w.b + 1];
+        seq_start = HSTU_CONST(int64_t, p.offsets)[w.b];
+        seq_end = HSTU_CONST(int64_t, p.offsets)[w.b + 1];
     } else {
-        seq_start = ((const int*)p.offsets)[w.b];
-        seq_end = ((const int*)p.offsets)[w.b + 1];
+        seq_start = HSTU_CONST(int, p.offsets)[w.b];
+        seq_end = HSTU_CONST(int, p.offsets)[w.b + 1];
     }
     // Values read from memory are the same for every lane; say so, so that everything derived from
     // them (loop bounds, tile classes, base addresses) lives in scalar registers.
@@ -280,7 +284,7 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
     if (n <= 0 || w.m0 >= w.nq || w.rbase < 0) return false;
 
     int t = 0;
-    if (p.targets) t = p.targets_i64 ? (int)((const int64_t*)p.targets)[w.b] : ((const int*)p.targets)[w.b];
+    if (p.targets) t = p.targets_i64 ? (int)HSTU_CONST(int64_t, p.targets)[w.b] : HSTU_CONST(int, p.targets)[w.b];
     t = __builtin_amdgcn_readfirstlane(t);
     SeqMask& M = w.M;
     M.n = n;
@@ -340,9 +344,12 @@ struct RowMask {
 // p = t * rcp(1 + exp2(t)) (TT::silu) and leaves the constant 1/c1 to the output scale.  p is zeroed where
 // the mask says so, rounded to the operand type and packed as two MFMA B operands.
 // `sp0` is the sequence position of this lane's first kv slot of the block.
-template <class TT, bool MASKED>
+// MASK: 0 = every pair valid, 1 = exact general predicate, 2 = plain causal (no window, targets or
+// contextual prefix: key position <= row position), which costs a compare and a select per element.
+template <class TT, int MASK>
 __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], float c1, const SeqMask& M,
                                           const RowMask& row, int sp0) {
+    const int causal_room = row.pos - sp0;  // a key at offset d from sp0 is visible iff d <= causal_room
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         // eight elements at a time, fenced, so that the scheduler cannot pile up temporaries of all sixteen
@@ -351,7 +358,8 @@ __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (
         for (int j = 0; j < 8; ++j) {
             const int r = half * 8 + j;
             float pr = TT::silu(s[r], c1);
-            if (MASKED) pr = row.valid(M, sp0 + 8 * (r >> 2) + (r & 3)) ? pr : 0.f;
+            if (MASK == 1) pr = row.valid(M, sp0 + 8 * (r >> 2) + (r & 3)) ? pr : 0.f;
+            if (MASK == 2) pr = (8 * (r >> 2) + (r & 3) <= causal_room) ? pr : 0.f;
             p[j] = pr;
         }
         pb[half] = TT::pack8(p);

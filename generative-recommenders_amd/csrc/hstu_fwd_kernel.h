@@ -9,7 +9,7 @@ namespace hstu {
 
 // One kv tile for one wave: S^T = K Q^T, P^T = s*sigmoid(alpha s) (masked if MASKED), O^T += V^T P^T.
 // `sp0` is the sequence position of this lane's first kv slot: tile start + 4*(lane/32).
-template <class TT, int DQK, int DV, int QT, int BN, bool MASKED>
+template <class TT, int DQK, int DV, int QT, int BN, int MASKED>
 __device__ __forceinline__ void tile_compute(const char* kt, const char* vt, const typename TT::vec8 (&qreg)[QT][DQK / 16],
                                              f32x16_t (&oacc)[DV / 32][QT], const int (&kaddr)[DQK / 16],
                                              const int (&vaddr)[2][DV / 32], float c1, const SeqMask& M, int sp0,
@@ -126,9 +126,9 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
         const int cls = M.classify(wR0, wR1, jt * BN, BN);
         const char* kt = smem + stage * STAGE;
         if (cls == 2) {
-            tile_compute<TT, DQK, DV, QT, BN, false>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
+            tile_compute<TT, DQK, DV, QT, BN, 0>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
         } else if (cls == 1) {
-            tile_compute<TT, DQK, DV, QT, BN, true>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
+            tile_compute<TT, DQK, DV, QT, BN, 1>(kt, kt + KTILE, qreg, oacc, kaddr, vaddr, p.c1, M, jt * BN + 4 * g, rows);
         }
         jt = jn;
         stage ^= 1;

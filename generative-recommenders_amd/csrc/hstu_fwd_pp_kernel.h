@@ -127,6 +127,9 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     // This kernel walks the contiguous tile range [jt_begin, jt_end): a tile inside it that holds no valid
     // pair (other targets' columns of a target row block) is computed and masked to zero rather than
     // skipped, which keeps the step count known up front and the loop free of side exits.
+    // no window, contextual prefix or targets: the mask of a diagonal tile is just "key <= row" (rows of the
+    // last, partly filled row block that lie past the sequence end are never stored, so they need no mask)
+    const bool plain_causal = p.w == 0 && p.c == 0 && p.targets == nullptr;
     const int jt_end = W.jt_end;
     const int T = jt_end - W.jt_begin;  // steps
     if (T <= 0) return;  // cannot happen for a row block with rows (each row sees itself); kept for safety
@@ -144,16 +147,15 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     constexpr int NPW = KCopy::PER_WAVE + VCopy::PER_WAVE;  // copy instructions per wave and step
     static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
 
-    // Copy schedule.  With 3 slots, step i copies V(i+1) and K(i+2) and its end waits for the copies of step
-    // i-1; before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1.  With 2 slots, step i copies
-    // V(i) and K(i+1) and waits for them at its own end; before step 0 only K(t0) is copied.
+    // Copy schedule.  Before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1.  With 3 slots,
+    // step i copies V(i+1) and K(i+2) and its end waits for the copies of step i-1.  With 2 slots, step i >= 1
+    // copies V(i) and K(i+1) and waits for them at its own end (step 0 copies nothing: its tiles came with
+    // the prologue, so that the first steps of a workgroup do not each expose a memory latency).
     constexpr int AHEAD = NSLOT - 2;  // 1 or 0
     if (grp == 0) {
         kcopy.issue(kbase, k_rsb, t_cur * BN, n, smem, wave);
-        if (NSLOT == 3) {
-            vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
-            kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
-        }
+        vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
+        kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
     }
 
     vec8 qreg[KS];
@@ -274,10 +276,13 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     auto valu_phase = [&](int tile) __attribute__((always_inline)) {
         if (tile >= full_begin && tile < full_end) {
 #pragma unroll
-            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, false>(s[sub], pb[sub], p.c1, M, row, 0);
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, 0>(s[sub], pb[sub], p.c1, M, row, 0);
+        } else if (plain_causal) {
+#pragma unroll
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, 2>(s[sub], pb[sub], p.c1, M, row, tile * BN + 4 * g + sub * 32);
         } else {
 #pragma unroll
-            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, true>(s[sub], pb[sub], p.c1, M, row, tile * BN + 4 * g + sub * 32);
+            for (int sub = 0; sub < NS; ++sub) silu_pack<TT, 1>(s[sub], pb[sub], p.c1, M, row, tile * BN + 4 * g + sub * 32);
         }
     };
     auto end_of_step = [&]() __attribute__((always_inline)) {
@@ -305,8 +310,10 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
             end_of_step();
             ++t_cur;
         };
+        if (NSLOT == 3) {
 #pragma unroll
-        for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
+            for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
+        }
         gemm1_only(0);
         if (NG == 2) __syncthreads();
         valu_phase(t_cur);
