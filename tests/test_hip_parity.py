@@ -408,3 +408,55 @@ def test_sort_by_length_changes_only_the_schedule(pkg, dev, cfg):
     torch.cuda.synchronize()
     assert torch.equal(a, b)
     assert_parity(a, _ref_full(q, k, v, offs, t, 2304, 0.09, 500, 0), "sorted")
+
+
+def _random_case(seed):
+    rng = np.random.default_rng(seed)
+    B = int(rng.integers(1, 7))
+    D = int(rng.choice([32, 64, 128]))
+    H = int(rng.choice([1, 2, 3]))
+    c = int(rng.choice([0, 0, 1, 5, 70]))
+    w = int(rng.choice([0, 0, 1, 17, 64, 200, 1000]))
+    f = int(rng.choice([0, 0, 0, 3, 40])) if w > 0 else 0
+    has_t = bool(rng.integers(0, 2))
+    hi = int(rng.choice([40, 130, 300, 700]))
+    uih = rng.integers(0, hi + 1, size=B)
+    tg = rng.integers(0, int(rng.choice([1, 5, 90])) + 1, size=B) if has_t else np.zeros(B, dtype=np.int64)
+    lengths = uih + tg + c
+    delta = 0
+    if rng.random() < 0.3:
+        delta = int(rng.integers(1, 70))
+        lengths = np.maximum(lengths, delta + c)
+        tg = np.minimum(tg, lengths - c)
+        f = 0  # delta_hstu_mha has no min_full_attn_seq_len argument
+    N = int(lengths.max()) + int(rng.integers(0, 40))
+    return dict(seed=seed, B=B, D=D, H=H, c=c, w=w, f=f, has_t=has_t, lengths=lengths, tg=tg, delta=delta, N=max(N, 1),
+                cfg=int(rng.choice([1, 2, 3])), dtype=[torch.bfloat16, torch.float16][int(rng.integers(0, 2))])
+
+
+@pytest.mark.parametrize("seed", list(range(7000, 7080)))
+def test_random_parameter_sweep(pkg, dev, seed):
+    """Random draws over every argument of both entry points (mask parameters, ragged lengths, delta, dims,
+    kernels), small enough that the oracle takes milliseconds."""
+    p = _random_case(seed)
+    _announce("random", {k: (v.tolist() if isinstance(v, np.ndarray) else v) for k, v in p.items()})
+    q, k, v, offs, t = make_case(seed, p["lengths"], p["H"], p["D"], targets=p["tg"], dtype=p["dtype"],
+                                 delta_size=p["delta"])
+    if p["dtype"] == torch.float16:
+        v.mul_(1024.0)  # keep fp16 outputs out of the subnormal range (the op is linear in v)
+    if not p["has_t"]:
+        t = None
+    alpha = 1.0 / p["D"] ** 0.5
+    if int(p["lengths"].sum()) == 0:
+        return
+    if p["delta"] > 0:
+        got = pkg.delta_hstu_mha(
+            p["N"], alpha, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=None if t is None else t.to(dev),
+            max_attn_len=p["w"], contextual_seq_len=p["c"], tile_config=p["cfg"],
+        )
+        torch.cuda.synchronize()
+        ref = O.cached_hstu_mha_per_sequence(p["N"], alpha, q.float(), k.float(), v.float(), offs, t, p["w"], p["c"])
+    else:
+        got = _run_full(pkg, dev, q, k, v, offs, t, p["N"], alpha, p["w"], p["c"], p["f"], p["cfg"])
+        ref = _ref_full(q, k, v, offs, t, p["N"], alpha, p["w"], p["c"], p["f"])
+    assert_parity(got, ref, str(p["seed"]))
