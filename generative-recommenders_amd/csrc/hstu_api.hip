@@ -130,6 +130,21 @@ int launch_dim(const hstu::FwdParams& p, int d, int cfg, int rows_per_pair, int 
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
 
+// 1 if the current device is gfx950, 0 if not, cached per device ordinal (the kernels use gfx950-only
+// instructions; the reference's native op makes the same kind of check, flash_common.cpp:420-422).
+int current_device_is_gfx950() {
+    static int cache[64];  // 0 unknown, 1 yes, 2 no; racing threads store the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    if (dev < 0 || dev >= 64) return 0;
+    if (cache[dev] == 0) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+        cache[dev] = strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 2;
+    }
+    return cache[dev] == 1;
+}
+
 }  // namespace
 
 extern "C" {
@@ -196,6 +211,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     int rc = hstu_hip_check_args(a);
     if (rc != HSTU_OK) return rc;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;
+    if (!current_device_is_gfx950()) return HSTU_ERR_BAD_DEVICE;
     hipStream_t stream = (hipStream_t)stream_;
 
     hstu::FwdParams p;
