@@ -32,7 +32,7 @@ def run_gpu(wl, args, pkg, workloads, torch):
     inp = workloads.make_inputs(wl, dev, fused_buffer=args.fused_buffer)
     q, k, v = inp["q"], inp["k"], inp["v"]
     kw = dict(num_targets=inp["num_targets"], max_attn_len=wl.max_attn_len, contextual_seq_len=wl.contextual_seq_len,
-              tile_config=args.tile_config)
+              tile_config=args.tile_config, kv_splits=args.kv_splits)
     sort_kw = dict(sort_by_length=not args.no_sort)  # the reference's bench sets the same hint for its native path
     scales = {}
     if wl.dtype == "fp8":
@@ -116,6 +116,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="headline")
     ap.add_argument("--tile-config", type=int, default=0)
+    ap.add_argument("--kv-splits", type=int, default=0, help="0 = the library's own rule, 1 = off, 2..8 = forced")
     ap.add_argument("--fused-buffer", action="store_true", help="q/k/v as column slices of one [L,H,3D] buffer")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sort", action="store_true", help="do not pass sort_by_length=True to hstu_mha")
@@ -158,9 +159,12 @@ def main():
         peak = PEAK_TFLOPS[wl.dtype]
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
-    auto_cfg = 2 if (wl.delta_size == 0 and wl.total_kv // wl.batch >= 3072) else 3  # the library's own rule
-    cfg = args.tile_config or auto_cfg
+    cfg, splits = pkg.ops.hip_backend.plan_for(
+        batch=wl.batch, heads=wl.heads, dqk=wl.dqk, dv=wl.dv, total_q=wl.batch * wl.delta_size if wl.delta_size else wl.total_kv,
+        total_kv=wl.total_kv, max_seq_len=wl.max_seq_len, delta_size=wl.delta_size, tile_config=args.tile_config,
+        kv_splits=args.kv_splits, sort_by_length=wl.delta_size == 0 and not args.no_sort)
     roof["kernel"] = {1: "hstu_fwd_kernel", 2: "hstu_fwd_pp_kernel<NG=2>", 3: "hstu_fwd_pp_kernel<NG=1>"}[cfg]
+    roof["kv_splits"] = splits
     roof["kernel_ms"] = round(ev_ms, 4)
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = nbytes
@@ -182,7 +186,7 @@ def main():
             "batch": wl.batch, "heads": wl.heads, "dqk": wl.dqk, "dv": wl.dv, "max_seq_len": wl.max_seq_len,
             "total_tokens": wl.total_kv, "max_attn_len": wl.max_attn_len, "contextual_seq_len": wl.contextual_seq_len,
             "num_targets": wl.num_targets is not None, "delta_size": wl.delta_size,
-            "tile_config": args.tile_config, "fused_buffer": args.fused_buffer,
+            "tile_config": args.tile_config, "kv_splits": args.kv_splits, "fused_buffer": args.fused_buffer,
         },
         "pct_mfma_peak": round(100.0 * tflops / PEAK_TFLOPS[wl.dtype], 2),
         "reference_convention_tflops": round(ref_flops / (ev_ms * 1e-3) / 1e12, 2),

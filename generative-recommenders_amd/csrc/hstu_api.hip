@@ -85,11 +85,12 @@ int launch(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
 }
 
 template <class TT, int DQK, int DV, int BN, int NG>
-int launch_pp(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
+int launch_pp(const hstu::FwdParams& p0, int num_pairs, int64_t total_q, hipStream_t stream) {
     constexpr int smem = 0;  // the kernel's LDS is a static array
     auto kern = hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN, NG>;
     const int pairs_per_xcd = (num_pairs + 7) / 8;
-    const long long grid = (long long)pairs_per_xcd * 8 * p0.num_mb;
+    const int splits = p0.kv_splits > 1 ? p0.kv_splits : 1;
+    const long long grid = (long long)pairs_per_xcd * 8 * p0.num_mb * splits;
     if (grid <= 0) return HSTU_OK;
     if (grid > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     hstu::FwdParams p = p0;
@@ -100,32 +101,103 @@ int launch_pp(const hstu::FwdParams& p0, int num_pairs, hipStream_t stream) {
         set_last_error("kernel launch", e);
         return HSTU_ERR_LAUNCH;
     }
+    if (splits > 1) {
+        const long long threads = (long long)total_q * p.H * (DV / 4);
+        const long long blocks = (threads + 255) / 256;
+        if (blocks > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+        hipLaunchKernelGGL(hstu::hstu_reduce_splits_kernel<typename TT::out_elem>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                           p, total_q, DV, NG * 128);
+        e = hipGetLastError();
+        if (e != hipSuccess) {
+            set_last_error("reduce kernel launch", e);
+            return HSTU_ERR_LAUNCH;
+        }
+    }
     return HSTU_OK;
 }
 
 template <class TT, int D>
-int launch_cfg(const hstu::FwdParams& p0, int cfg, int rows_per_pair, int num_pairs, hipStream_t stream) {
+int launch_cfg(const hstu::FwdParams& p0, int cfg, int rows_per_pair, int num_pairs, int64_t total_q, hipStream_t stream) {
     hstu::FwdParams p = p0;
     if (cfg == 2) {
         p.num_mb = (rows_per_pair + 255) / 256;
-        return launch_pp<TT, D, D, 64, 2>(p, num_pairs, stream);
+        return launch_pp<TT, D, D, 64, 2>(p, num_pairs, total_q, stream);
     }
     if (cfg == 3) {
         p.num_mb = (rows_per_pair + 127) / 128;
-        return launch_pp<TT, D, D, 64, 1>(p, num_pairs, stream);
+        return launch_pp<TT, D, D, 64, 1>(p, num_pairs, total_q, stream);
     }
     p.num_mb = (rows_per_pair + 127) / 128;
     return launch<TT, D, D, 1, 4, 64, 2>(p, num_pairs, stream);
 }
 
 template <class TT>
-int launch_dim(const hstu::FwdParams& p, int d, int cfg, int rows_per_pair, int num_pairs, hipStream_t stream) {
+int launch_dim(const hstu::FwdParams& p, int d, int cfg, int rows_per_pair, int num_pairs, int64_t total_q,
+               hipStream_t stream) {
     switch (d) {
-        case 32: return launch_cfg<TT, 32>(p, cfg, rows_per_pair, num_pairs, stream);
-        case 64: return launch_cfg<TT, 64>(p, cfg, rows_per_pair, num_pairs, stream);
-        case 128: return launch_cfg<TT, 128>(p, cfg, rows_per_pair, num_pairs, stream);
+        case 32: return launch_cfg<TT, 32>(p, cfg, rows_per_pair, num_pairs, total_q, stream);
+        case 64: return launch_cfg<TT, 64>(p, cfg, rows_per_pair, num_pairs, total_q, stream);
+        case 128: return launch_cfg<TT, 128>(p, cfg, rows_per_pair, num_pairs, total_q, stream);
         default: return HSTU_ERR_BAD_HEAD_DIM;
     }
+}
+
+// What a call will do, from sizes the host knows without reading the offsets.
+struct Plan {
+    int cfg;               // tile configuration, 1-based
+    int splits;            // workgroups per row block along kv (1 = no split)
+    int chunk;             // kv tiles per run when split
+    size_t order_bytes;    // sequence ranking, at the start of the workspace
+    size_t counts_bytes;   // runs per row block, behind the ranking
+    size_t partial_bytes;  // fp32 partial outputs of the runs, 256-byte aligned behind the counts
+    size_t total() const { return order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0); }
+};
+
+constexpr int kMaxSplits = 8;
+constexpr int kTileRows = 64;  // kv rows per tile of every configuration
+
+Plan make_plan(const HstuFwdArgs* a) {
+    Plan pl = {0, 1, 0, 0, 0, 0};
+    // The ping-pong kernel (256-row blocks, one workgroup per CU) wins when the average sequence is long; the
+    // one-group pipeline (128-row blocks, two workgroups per CU) wastes less on short or very uneven sequences
+    // and in delta mode.
+    pl.cfg = a->tile_config;
+    const long long avg_tiles = a->batch > 0 ? a->total_kv / a->batch / kTileRows : 0;
+    if (pl.cfg == 0) {
+        if (a->delta_size == 0) {
+            pl.cfg = avg_tiles >= 3072 / kTileRows ? 2 : 3;
+        } else {
+            // few long histories: 256-row blocks, whose kv range is then split below so that every CU gets one
+            const long long blocks256 = (long long)a->batch * a->heads * ((a->delta_size + 255) / 256);
+            pl.cfg = (blocks256 * 2 <= 256 && avg_tiles >= 32) ? 2 : 3;
+        }
+    }
+    if (a->sort_by_length && a->batch >= 2 && a->batch <= kMaxSortBatch) pl.order_bytes = (size_t)a->batch * sizeof(int);
+    if (pl.cfg < 2 || a->batch <= 0) return pl;
+    const int bm = pl.cfg == 2 ? 256 : 128;
+    const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
+    const long long blocks = (long long)a->batch * a->heads * ((rows_per_pair + bm - 1) / bm);
+    const int max_tiles = (a->max_seq_len + kTileRows - 1) / kTileRows;
+    int s = 1;
+    if (a->kv_splits > 0) {
+        s = a->kv_splits;
+    } else if (a->delta_size > 0) {
+        // Delta mode has few query rows per sequence: with a small batch the row blocks alone do not fill the
+        // 256 CUs.  Cut the kv range so that the chip is just filled (more runs than that only add partial-sum
+        // traffic: with every CU busy the clock drops and the time per tile rises), in runs of at least 16 tiles.
+        const long long resident = pl.cfg == 2 ? 256 : 512;  // workgroups the chip holds at once
+        long long want = resident / blocks;
+        if (want > max_tiles / 16) want = max_tiles / 16;
+        if (want > kMaxSplits) want = kMaxSplits;
+        if (want >= 2) s = (int)want;
+    }
+    if (s > 1) {
+        pl.splits = s;
+        pl.chunk = (max_tiles + s - 1) / s;
+        pl.counts_bytes = (size_t)blocks * sizeof(int);
+        pl.partial_bytes = (size_t)s * (size_t)a->total_q * a->heads * a->dv * sizeof(float);
+    }
+    return pl;
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -170,8 +242,18 @@ const char* hstu_hip_status_string(int status) {
 const char* hstu_hip_last_error(void) { return g_last_error; }
 
 size_t hstu_hip_workspace_bytes(const HstuFwdArgs* a) {
-    if (!a || !a->sort_by_length || a->batch < 2 || a->batch > kMaxSortBatch) return 0;
-    return (size_t)a->batch * sizeof(int);
+    if (!a || a->batch <= 0 || a->heads <= 0 || a->total_q <= 0) return 0;
+    return make_plan(a).total();
+}
+
+int hstu_hip_plan(const HstuFwdArgs* a, int32_t* tile_config, int32_t* kv_splits) {
+    int rc = hstu_hip_check_args(a);
+    if (rc != HSTU_OK) return rc;
+    Plan pl = make_plan(a);
+    if (pl.splits > 1 && !(a->workspace && (size_t)a->workspace_bytes >= pl.total()) && a->kv_splits <= 1) pl.splits = 1;
+    if (tile_config) *tile_config = pl.cfg;
+    if (kv_splits) *kv_splits = pl.splits;
+    return HSTU_OK;
 }
 
 int hstu_hip_tile_configs(void) { return kNumConfigs; }
@@ -191,6 +273,7 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     if (a->delta_size == 0 && a->total_q != a->total_kv) return HSTU_ERR_BAD_SHAPE;
     if (a->total_kv > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     if (a->tile_config < 0 || a->tile_config > kNumConfigs) return HSTU_ERR_BAD_SHAPE;
+    if (a->kv_splits < 0 || a->kv_splits > kMaxSplits || (a->kv_splits > 1 && a->tile_config == 1)) return HSTU_ERR_BAD_SHAPE;
     if (a->workspace && (a->workspace_bytes < 0 || (reinterpret_cast<uintptr_t>(a->workspace) & 3) != 0)) return HSTU_ERR_MISALIGNED;
     if (a->dqk != a->dv) return HSTU_ERR_BAD_HEAD_DIM;  // as the reference's native op, flash_common.cpp:543-545
     if (a->dqk != 32 && a->dqk != 64 && a->dqk != 128) return HSTU_ERR_BAD_HEAD_DIM;
@@ -248,9 +331,25 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
         p.oscale *= a->v_scale / hstu::Fp8::PSCALE;
     }
 
+    // Both uses of the caller's scratch memory are optimisations that never change the result: without enough of
+    // it an automatic choice falls back to the plain schedule, an explicit kv_splits > 1 is an error.
+    Plan plan = make_plan(a);
+    const bool ws_ok = a->workspace && (size_t)a->workspace_bytes >= plan.total();
+    if (plan.splits > 1 && !ws_ok) {
+        if (a->kv_splits > 1) return a->workspace ? HSTU_ERR_BAD_SHAPE : HSTU_ERR_NULL_POINTER;
+        plan.splits = 1;
+        plan.partial_bytes = plan.counts_bytes = 0;
+    }
+    if (plan.splits > 1) {
+        char* base = (char*)a->workspace + plan.order_bytes;
+        p.split_counts = (int*)base;
+        p.partial = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(base + plan.counts_bytes) + 255) & ~(uintptr_t)255);
+        p.partial_stride = (int64_t)a->total_q * a->heads * a->dv;
+        p.kv_chunk = plan.chunk;
+    }
+    p.kv_splits = plan.splits;
     // optional schedule: rank the sequences by length into the caller's scratch memory
-    const size_t ws_need = hstu_hip_workspace_bytes(a);
-    if (ws_need > 0 && a->workspace && (size_t)a->workspace_bytes >= ws_need) {
+    if (plan.order_bytes > 0 && a->workspace && (size_t)a->workspace_bytes >= plan.order_bytes) {
         int* order = (int*)a->workspace;
         hipLaunchKernelGGL(hstu::hstu_rank_kernel, dim3((a->batch + 255) / 256), dim3(256), 0, stream, a->seq_offsets,
                            a->seq_offsets_i64, a->batch, order);
@@ -266,14 +365,10 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     const long long num_pairs_ll = (long long)a->batch * a->heads;
     if (num_pairs_ll > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     const int num_pairs = (int)num_pairs_ll;
-    // Automatic choice, from sizes the host knows without reading the offsets: the ping-pong kernel (256-row
-    // blocks, one workgroup per CU) wins when the average sequence is long; the one-group pipeline (128-row
-    // blocks, two workgroups per CU) wastes less on short or very uneven sequences and in delta mode.
-    int cfg = a->tile_config;
-    if (cfg == 0) cfg = (a->delta_size == 0 && a->total_kv / a->batch >= 3072) ? 2 : 3;
-    if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
-    if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
-    return launch_dim<hstu::Fp8>(p, a->dqk, cfg, rows_per_pair, num_pairs, stream);
+    const int cfg = plan.cfg;
+    if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, rows_per_pair, num_pairs, a->total_q, stream);
+    if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, rows_per_pair, num_pairs, a->total_q, stream);
+    return launch_dim<hstu::Fp8>(p, a->dqk, cfg, rows_per_pair, num_pairs, a->total_q, stream);
 }
 
 }  // extern "C"

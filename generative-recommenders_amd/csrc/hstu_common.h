@@ -67,6 +67,16 @@ struct FwdParams {
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
     float c1;           // -alpha * log2(e): Q is multiplied by it when loaded
     float oscale;       // (alpha / max_seq_len) / c1 = -1 / (max_seq_len * log2(e)); 0 if alpha == 0
+    // Split of the kv range of a row block into runs of `kv_chunk` tiles, each taken by its own workgroup; the
+    // grid holds `kv_splits` workgroups per row block (1 = off) and those past the end of a short range exit at
+    // once.  Each run writes its unscaled fp32 accumulators to partial[split][row][head][dv] (dense) and run 0
+    // writes the number of runs to split_counts[(b * H + h) * num_mb + row block]; a second kernel adds the
+    // runs in a fixed order.
+    int kv_splits;
+    int kv_chunk;
+    float* partial;
+    int64_t partial_stride;  // floats per split = total_q * H * dv
+    int* split_counts;
 };
 
 // Element types.  ES = bytes per element; `vec8` = eight elements = one MFMA operand of a lane;
@@ -222,6 +232,9 @@ struct Work {
     int m0;           // first query row of the workgroup (index into the nq rows)
     int rbase;        // sequence position of query row 0 (n - delta_size in delta mode)
     int u;            // number of non-target positions
+    int split;        // which run of the kv range this workgroup takes (0 when the range is not split)
+    int nsplit;       // number of non-empty runs of this row block
+    int block_id;     // (b * H + h) * num_mb + row block
     int R0, R1;       // sequence positions of the workgroup's first and last row (inclusive)
     int jt_begin;     // first kv tile that can hold a valid pair
     int jt_end;       // one past the last such tile
@@ -236,7 +249,14 @@ template <int BM, int BN>
 __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
     const int bid = blockIdx.x;
     const int xcd = bid & 7;
-    const int slot = bid >> 3;
+    int slot = bid >> 3;
+    // the splits of one row block are neighbours on one XCD
+    w.split = 0;
+    if (p.kv_splits > 1) {
+        const int s0 = slot / p.kv_splits;
+        w.split = slot - s0 * p.kv_splits;
+        slot = s0;
+    }
     // Heaviest work first.  Within a pair that is the last row block -- except that with a contextual prefix
     // the first row block (its contextual rows see every non-target key) is the heaviest of all and runs
     // many times longer than the others, so the first row blocks of all pairs are launched before anything else.
@@ -308,6 +328,15 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
     if (p.w > 0 && p.f == 0 && !ctx_rows && idr_lo - p.w > 0) kv_lo = idr_lo - p.w + M.shift;
     w.jt_end = (kv_hi + BN - 1) / BN;
     w.jt_begin = kv_lo / BN;
+    w.nsplit = 1;
+    w.block_id = (w.b * p.H + w.h) * p.num_mb + mb;
+    if (p.kv_splits > 1) {
+        w.nsplit = (w.jt_end - w.jt_begin + p.kv_chunk - 1) / p.kv_chunk;
+        const int b = w.jt_begin + w.split * p.kv_chunk;
+        if (b >= w.jt_end) return false;  // a short range has fewer runs than the grid provides
+        w.jt_end = b + p.kv_chunk < w.jt_end ? b + p.kv_chunk : w.jt_end;
+        w.jt_begin = b;
+    }
     w.skip_scan = p.w > 0 || p.c > 0 || p.targets != nullptr;
     return true;
 }
@@ -469,6 +498,72 @@ __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int
             for (int i = 0; i < 4; ++i) o4[i] = (elem)(oacc[dt][qt][r4 * 4 + i] * oscale);
             *(elem4*)(op + (dt * 32 + r4 * 8) * 2) = o4;
         }
+}
+
+// Unscaled fp32 accumulators of one block of 32 query rows to partial[split][row][head][dv]; 16 bytes per store.
+template <int DT, int QT>
+__device__ __forceinline__ void store_partial(const f32x16_t (&oacc)[DT][QT], int qt, float* partial, int64_t orow0, int ql,
+                                              int nq, int H, int h, int g) {
+    if (ql >= nq) return;
+    float* op = partial + ((orow0 + ql) * H + h) * (int64_t)(DT * 32) + g * 4;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            f32x4_t o4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o4[i] = oacc[dt][qt][r4 * 4 + i];
+            *(f32x4_t*)(op + dt * 32 + r4 * 8) = o4;
+        }
+}
+
+// out = oscale * (sum of the runs of the row's row block), rounded once; one thread per 4 consecutive dv.
+// The thread finds its sequence (delta mode: row / delta; otherwise a binary search of the offsets), skips
+// rows the forward kernel does not produce (past max_seq_len, or a sequence shorter than delta) and reads the
+// number of runs that run 0 of its row block recorded.
+template <class ELEM>
+__global__ __launch_bounds__(256) void hstu_reduce_splits_kernel(const FwdParams p, int64_t total_q, int dv, int bm) {
+    typedef __attribute__((ext_vector_type(4))) ELEM elem4;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over total_q * H * dv / 4
+    const int dv4 = dv >> 2;
+    if (idx >= total_q * p.H * dv4) return;
+    const int c = (int)(idx % dv4);
+    const int64_t rh = idx / dv4;
+    const int h = (int)(rh % p.H);
+    const int64_t row = rh / p.H;
+    auto offset = [&](int j) -> int64_t {
+        return p.offsets_i64 ? ((const int64_t*)p.offsets)[j] : (int64_t)((const int*)p.offsets)[j];
+    };
+    int b, r;
+    if (p.delta > 0) {
+        b = (int)(row / p.delta);
+        r = (int)(row - (int64_t)b * p.delta);
+        int64_t n = offset(b + 1) - offset(b);
+        if (n > p.max_seq_len) n = p.max_seq_len;
+        if (n <= 0 || n < p.delta) return;
+    } else {
+        int lo = 0, hi = p.B;  // last b with offsets[b] <= row
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (offset(mid) <= row) lo = mid; else hi = mid;
+        }
+        b = lo;
+        const int64_t start = offset(b);
+        int64_t n = offset(b + 1) - start;
+        if (n > p.max_seq_len) n = p.max_seq_len;
+        if (row - start >= n) return;
+        r = (int)(row - start);
+    }
+    const int runs = p.split_counts[(b * p.H + h) * p.num_mb + r / bm];
+    f32x4_t acc = *(const f32x4_t*)(p.partial + idx * 4);
+    for (int s = 1; s < runs; ++s) {
+        const f32x4_t x = *(const f32x4_t*)(p.partial + s * p.partial_stride + idx * 4);
+        acc += x;
+    }
+    elem4 o4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o4[i] = (ELEM)(acc[i] * p.oscale);
+    *(elem4*)(p.o + (row * p.o_rs + (int64_t)h * p.o_hs) * 2 + c * 8) = o4;
 }
 
 // Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit

@@ -132,6 +132,8 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     const bool plain_causal = p.w == 0 && p.c == 0 && p.targets == nullptr;
     const int jt_end = W.jt_end;
     const int T = jt_end - W.jt_begin;  // steps
+    const int64_t orow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
+    float* const my_partial = p.kv_splits > 1 ? p.partial + (int64_t)W.split * p.partial_stride : nullptr;
     if (T <= 0) return;  // cannot happen for a row block with rows (each row sees itself); kept for safety
     int t_cur = W.jt_begin;
 
@@ -367,8 +369,11 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     // the redundant copies of the last steps may still be in flight: they must land before the LDS is released
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
-    const int64_t orow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
-    store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
+    if (my_partial) {
+        store_partial<DT>(oacc, 0, my_partial, orow0, wq0 + l32, nq, p.H, W.h, g);
+        if (W.split == 0 && threadIdx.x == 0) p.split_counts[W.block_id] = W.nsplit;
+    } else
+        store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
 }
 
 }  // namespace hstu

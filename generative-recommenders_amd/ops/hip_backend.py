@@ -51,6 +51,7 @@ class HstuFwdArgs(ctypes.Structure):
         ("sort_by_length", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
+        ("kv_splits", ctypes.c_int32),
     ]
 
 
@@ -61,6 +62,7 @@ EXPORTS = (
     "hstu_hip_check_args",
     "hstu_hip_mha_fwd",
     "hstu_hip_workspace_bytes",
+    "hstu_hip_plan",
     "hstu_hip_tile_configs",
     "hstu_hip_tile_config_name",
 )
@@ -90,6 +92,8 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_check_args.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_mha_fwd.restype = ctypes.c_int
         L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
+        L.hstu_hip_plan.restype = ctypes.c_int
+        L.hstu_hip_plan.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
         L.hstu_hip_workspace_bytes.restype = ctypes.c_size_t
         L.hstu_hip_workspace_bytes.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_tile_configs.restype = ctypes.c_int
@@ -127,6 +131,27 @@ def tile_config_names() -> list:
     return [L.hstu_hip_tile_config_name(i + 1).decode() for i in range(L.hstu_hip_tile_configs())]
 
 
+def plan_for(batch, heads, dqk, dv, total_q, total_kv, max_seq_len, delta_size=0, tile_config=0, kv_splits=0,
+             sort_by_length=False, dtype=HSTU_BF16):
+    """(tile configuration, kv runs) the library would choose for a call of these sizes when given the workspace it
+    asks for.  Touches no device memory."""
+    a = HstuFwdArgs()
+    a.batch, a.heads, a.dqk, a.dv = batch, heads, dqk, dv
+    a.total_q, a.total_kv, a.max_seq_len, a.delta_size = total_q, total_kv, max_seq_len, delta_size
+    a.tile_config, a.kv_splits, a.sort_by_length, a.dtype = tile_config, kv_splits, 1 if sort_by_length else 0, dtype
+    # sizes only: the pointers are checked for presence and alignment, never followed
+    a.q = a.k = a.v = a.out = a.seq_offsets = 256
+    a.q_row_stride = a.k_row_stride = heads * dqk
+    a.v_row_stride = a.o_row_stride = heads * dv
+    a.q_head_stride = a.k_head_stride = dqk
+    a.v_head_stride = a.o_head_stride = dv
+    need = lib().hstu_hip_workspace_bytes(ctypes.byref(a))
+    a.workspace, a.workspace_bytes = (256, need) if need else (None, 0)
+    cfg, splits = ctypes.c_int32(0), ctypes.c_int32(0)
+    raise_for_status(lib().hstu_hip_plan(ctypes.byref(a), ctypes.byref(cfg), ctypes.byref(splits)))
+    return cfg.value, splits.value
+
+
 def _dtype_code(dt: torch.dtype) -> int:
     if dt == torch.bfloat16:
         return HSTU_BF16
@@ -155,6 +180,7 @@ def mha_fwd(
     v_scale: float = 1.0,
     tile_config: int = 0,
     sort_by_length: bool = False,
+    kv_splits: int = 0,
 ) -> None:
     """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors."""
     a = HstuFwdArgs()
@@ -186,6 +212,7 @@ def mha_fwd(
     a.q_scale, a.k_scale, a.v_scale = q_scale, k_scale, v_scale
     a.tile_config = tile_config
     a.sort_by_length = 1 if sort_by_length else 0
+    a.kv_splits = kv_splits
     workspace = None
     need = lib().hstu_hip_workspace_bytes(ctypes.byref(a))
     if need > 0:

@@ -9,7 +9,9 @@ messages and output shapes.  Differences, all explicit:
 * forward only -- inputs that require grad under ``torch.enable_grad()`` raise ``NotImplementedError``;
 * tensors must live on a HIP device; there is no CPU or PyTorch fallback;
 * fp8 (``torch.float8_e4m3fn``) q/k/v take per-tensor scales through ``q_scale``/``k_scale``/``v_scale``
-  and give bf16 output, as the reference's native op does (``flash_common.cpp:596-607``).
+  and give bf16 output, as the reference's native op does (``flash_common.cpp:596-607``);
+* ``tile_config`` / ``kv_splits`` choose the kernel and the split of the kv range over workgroups (0 = automatic);
+  they change the schedule, and with a split the fp32 summation order, never the mask or the scaling.
 """
 
 from typing import Optional
@@ -71,6 +73,7 @@ def hstu_mha(
     k_scale: float = 1.0,
     v_scale: float = 1.0,
     tile_config: int = 0,
+    kv_splits: int = 0,
 ) -> torch.Tensor:
     """Jagged HSTU attention forward; returns ``[L, H, Dv]``.
 
@@ -122,6 +125,7 @@ def hstu_mha(
         v_scale=v_scale,
         tile_config=tile_config,
         sort_by_length=sort_by_length,
+        kv_splits=kv_splits,
     )
     return out
 
@@ -142,6 +146,7 @@ def delta_hstu_mha(
     k_scale: float = 1.0,
     v_scale: float = 1.0,
     tile_config: int = 0,
+    kv_splits: int = 0,
 ) -> torch.Tensor:
     """Cached-KV (M-FALCON) forward: ``delta_q`` holds the last ``L // B`` positions of every sequence.
 
@@ -196,5 +201,6 @@ def delta_hstu_mha(
         k_scale=k_scale,
         v_scale=v_scale,
         tile_config=tile_config,
+        kv_splits=kv_splits,
     )
     return out

@@ -79,6 +79,14 @@ typedef struct HstuFwdArgs {
                                         4-byte aligned, owned by the caller, free to reuse once the call's work on
                                         `stream` has run */
     int64_t workspace_bytes;
+    int32_t kv_splits;               /* 0 = choose automatically (delta mode with too few row blocks to fill and
+                                        balance the chip is split when the workspace allows); 1 = never split;
+                                        S = 2..8: cut the kv range of every row block into runs of
+                                        ceil(ceil(max_seq_len / 64) / S) tiles of 64 rows, each run taken by its own
+                                        workgroup, and add the fp32 partial results in a second kernel.  Needs
+                                        `workspace`; tile configs 2 and 3 only.  The result is the same up to fp32
+                                        summation order.  The reference has no such option: its kernels run one
+                                        block per (sequence, head, row block) in both modes */
 } HstuFwdArgs;
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -109,6 +117,13 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* args, void* stream);
  * here the caller passes scratch memory, or NULL to run without the options that need it.
  */
 size_t hstu_hip_workspace_bytes(const HstuFwdArgs* args);
+
+/*
+ * The tile configuration and number of kv runs hstu_hip_mha_fwd would use for these arguments (either pointer may
+ * be NULL).  Returns what hstu_hip_check_args returns.  Diagnostic only: the reference picks its tile configuration
+ * with an autotuner at run time (ops/triton/triton_hstu_attention.py:1643), this library by a fixed rule.
+ */
+int hstu_hip_plan(const HstuFwdArgs* args, int32_t* tile_config, int32_t* kv_splits);
 
 /* Number of selectable tile configurations and a short name for each (1-based ids). */
 int hstu_hip_tile_configs(void);

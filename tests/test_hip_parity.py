@@ -219,6 +219,74 @@ def test_delta_against_oracle_and_tail_of_full(pkg, dev, delta, w, c, D, cfg):
     assert_parity(got, full[idx.to(dev)], "delta vs tail of full", rel_tol=2e-3)
 
 
+@pytest.mark.parametrize("cfg", [2, 3])
+@pytest.mark.parametrize("splits", [2, 3, 8])
+@pytest.mark.parametrize("delta,w,c,D", [(256, 0, 0, 128), (130, 50, 4, 64), (1, 0, 0, 32), (200, 0, 0, 128)])
+def test_delta_kv_splits(pkg, dev, delta, w, c, D, splits, cfg):
+    """The kv range of every row block cut over several workgroups: same result as the oracle and as the unsplit
+    kernel up to fp32 summation order.  Lengths start at delta + c, so short sequences leave some splits empty."""
+    _announce("delta kv_splits", delta, w, c, D, splits, cfg)
+    rng = np.random.default_rng(1000 + delta)
+    lengths = rng.integers(0, 1500, size=4) + delta + c
+    lengths[1] = delta + c
+    q, k, v, offs, t = make_case(77 + delta, lengths, 2, D, targets=[delta] * 4)
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(4)])
+    dq = q[idx].contiguous()
+    N = int(lengths.max())
+    alpha = 1.0 / D**0.5
+    args = (N, alpha, dq.to(dev), k.to(dev), v.to(dev), offs.to(dev))
+    kw = dict(num_targets=t.to(dev), max_attn_len=w, contextual_seq_len=c, tile_config=cfg)
+    got = pkg.delta_hstu_mha(*args, **kw, kv_splits=splits)
+    one = pkg.delta_hstu_mha(*args, **kw, kv_splits=1)
+    torch.cuda.synchronize()
+    ref = O.cached_hstu_mha_per_sequence(N, alpha, dq.float(), k.float(), v.float(), offs, t, w, c)
+    assert_parity(got, ref, "split vs oracle")
+    assert_parity(got, one, "split vs unsplit", rel_tol=2e-3)
+
+
+@pytest.mark.parametrize("cfg", [2, 3])
+def test_full_mode_kv_splits(pkg, dev, cfg):
+    """kv_splits also applies to hstu_mha (never chosen automatically there): ragged batch with every mask option."""
+    _announce("full kv_splits", cfg)
+    lengths = [1300, 0, 65, 700, 1]
+    q, k, v, offs, t = make_case(4242, lengths, 2, 64, targets=[10, 0, 3, 0, 0])
+    N, alpha = 1300, 0.125
+    for w, c, f in [(0, 0, 0), (300, 5, 0), (100, 0, 64)]:
+        ref = _ref_full(q, k, v, offs, t, N, alpha, w, c, f)
+        got = pkg.hstu_mha(
+            N, alpha, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev), max_attn_len=w,
+            contextual_seq_len=c, min_full_attn_seq_len=f, tile_config=cfg, kv_splits=4, sort_by_length=True,
+        )
+        torch.cuda.synchronize()
+        assert_parity(got, ref, f"w={w} c={c} f={f}")
+
+
+def test_kv_splits_rejections_and_auto(pkg, dev):
+    """Out-of-range or cfg-1 splits are shape errors; the automatic rule splits a small delta batch and leaves
+    a large one alone (seen through the workspace size)."""
+    import ctypes
+
+    from generative_recommenders_amd.ops import hip_backend as hb
+
+    _announce("kv_splits rejections")
+    q, k, v, offs, t = make_case(5, [300, 200], 2, 64)
+    with pytest.raises(ValueError):
+        pkg.hstu_mha(300, 0.1, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), kv_splits=9)
+    with pytest.raises(ValueError):
+        pkg.hstu_mha(300, 0.1, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), kv_splits=2, tile_config=1)
+    # 32 users x 4 heads x one 256-row block = 128 workgroups: 256-row kernel, two runs each
+    assert hb.plan_for(32, 4, 128, 128, 32 * 256, 32 * 3000, 4352, delta_size=256) == (2, 2)
+    # 512 users fill the chip on their own
+    assert hb.plan_for(512, 4, 128, 128, 512 * 256, 512 * 3000, 4352, delta_size=256) == (3, 1)
+    # short histories are not worth cutting
+    assert hb.plan_for(32, 4, 128, 128, 32 * 256, 32 * 600, 700, delta_size=256) == (3, 1)
+    a = hb.HstuFwdArgs()
+    a.batch, a.heads, a.dqk, a.dv, a.delta_size = 32, 4, 128, 128, 256
+    a.total_q, a.total_kv, a.max_seq_len = 32 * 256, 32 * 3000, 4352
+    need = hb.lib().hstu_hip_workspace_bytes(ctypes.byref(a))
+    assert need == 4 * 128 + 2 * a.total_q * 4 * 128 * 4 + 256  # run counts, two fp32 partial outputs, alignment slack
+
+
 def test_invariants_on_device(pkg, dev):
     """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
     permuting two targets permutes the outputs (stu_test.py:180-321)."""
@@ -384,6 +452,10 @@ def test_fp8_delta_and_scales(pkg, dev):
     ref = O.cached_hstu_mha_per_sequence(700, alpha, dq, k, v, offs, t)
     assert _cos(got.cpu(), ref) >= 0.995
     assert torch.equal(got.float(), half.float() * 2.0)
+    split = pkg.delta_hstu_mha(700, alpha, qq.to(dev), kq.to(dev), vq.to(dev), offs.to(dev), v_scale=vs, kv_splits=3, **kw)
+    torch.cuda.synchronize()
+    assert _cos(split.cpu(), ref) >= 0.995
+    assert_parity(split, got, "fp8 split vs unsplit", rel_tol=2e-3)
 
 
 @pytest.mark.parametrize("cfg", [1, 2, 3])
