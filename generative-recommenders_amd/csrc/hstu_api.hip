@@ -12,22 +12,28 @@
 
 namespace hstu {
 
-// order[rank] = sequence index, longest sequence first (ties by index).  One thread per sequence, each
-// counting the sequences that precede it; the offsets array is small and stays in cache.
+// order[rank] = sequence index, longest sequence first (ties by index).  One wave per sequence: its lanes
+// share out the other sequences and count, by ballot, those that precede it.
 __global__ __launch_bounds__(256) void hstu_rank_kernel(const void* offsets, int offsets_i64, int B, int* order) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= B) return;
     auto len = [&](int j) -> long long {
         return offsets_i64 ? ((const long long*)offsets)[j + 1] - ((const long long*)offsets)[j]
                            : (long long)(((const int*)offsets)[j + 1] - ((const int*)offsets)[j]);
     };
+    const int i = (blockIdx.x * 256 + threadIdx.x) >> 6;  // wave-uniform
+    const int lane = threadIdx.x & 63;
+    if (i >= B) return;
     const long long ni = len(i);
     int rank = 0;
-    for (int j = 0; j < B; ++j) {
-        const long long nj = len(j);
-        rank += (nj > ni) || (nj == ni && j < i);
+    for (int j0 = 0; j0 < B; j0 += 64) {
+        const int j = j0 + lane;
+        bool before = false;
+        if (j < B) {
+            const long long nj = len(j);
+            before = (nj > ni) || (nj == ni && j < i);
+        }
+        rank += __popcll(__ballot(before));
     }
-    order[rank] = i;
+    if (lane == 0) order[rank] = i;
 }
 
 }  // namespace hstu
@@ -351,7 +357,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     // optional schedule: rank the sequences by length into the caller's scratch memory
     if (plan.order_bytes > 0 && a->workspace && (size_t)a->workspace_bytes >= plan.order_bytes) {
         int* order = (int*)a->workspace;
-        hipLaunchKernelGGL(hstu::hstu_rank_kernel, dim3((a->batch + 255) / 256), dim3(256), 0, stream, a->seq_offsets,
+        hipLaunchKernelGGL(hstu::hstu_rank_kernel, dim3((a->batch + 3) / 4), dim3(256), 0, stream, a->seq_offsets,
                            a->seq_offsets_i64, a->batch, order);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) {
