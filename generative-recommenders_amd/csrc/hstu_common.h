@@ -62,6 +62,8 @@ struct FwdParams {
     const int* order;   // NULL, or sequence indices sorted by decreasing length (scheduling only)
     int num_mb;         // row blocks per (sequence, head) pair in the grid
     int pairs_per_xcd;  // ceil(B*H / 8)
+    int slots_per_xcd;  // work items per XCD = pairs_per_xcd * num_mb * kv_splits
+    int* queue;         // NULL, or 8 counters 64 bytes apart (one per XCD) handing out work items
     int max_seq_len;
     int delta;          // 0 = full attention
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
@@ -242,12 +244,11 @@ struct Work {
     SeqMask M;
 };
 
-// Decode blockIdx.x.  Workgroup ids go round-robin over the 8 XCDs, so ids congruent mod 8 share
-// an L2: all row blocks of one (sequence, head) pair stay on one XCD, heaviest block first.
-// Returns false if this workgroup has nothing to do.
+// Decode work item `bid` (the workgroup id in a one-item-per-workgroup launch).  Workgroup ids go round-robin
+// over the 8 XCDs, so ids congruent mod 8 share an L2: all row blocks of one (sequence, head) pair stay on one
+// XCD, heaviest block first.  Returns false if the item holds no work.
 template <int BM, int BN>
-__device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w) {
-    const int bid = blockIdx.x;
+__device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid) {
     const int xcd = bid & 7;
     int slot = bid >> 3;
     // the splits of one row block are neighbours on one XCD

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     const int l32 = lane & 31;    // operand row (A) / column (B, C) this lane holds
 
     Work W;
-    if (!decode_work<BM, BN>(p, W)) return;
+    if (!decode_work<BM, BN>(p, W, blockIdx.x)) return;
     const SeqMask& M = W.M;
     const int n = W.n, nq = W.nq;
 

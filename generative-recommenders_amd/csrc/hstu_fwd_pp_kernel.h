@@ -74,7 +74,7 @@ struct TileCopy {
 //         barrier per tile); the overlap of matrix and VALU work then comes from the two workgroups that share a
 //         CU.  It wastes less on short sequences, whose last 256-row block would be mostly empty.
 template <class TT, int DQK, int DV, int BN, int NG>
-__global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParams p) {
+__global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParams p_arg) {
     typedef typename TT::vec8 vec8;
     static_assert(DQK == DV, "the interleaved matrix phase assumes as many first-product as second-product MFMAs");
     static_assert(NG == 1 || NG == 2, "one or two wave groups");
@@ -88,7 +88,9 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     constexpr int NSLOT = NG == 2 ? 3 : 2;
     // LDS: NSLOT K slots, then NSLOT V slots.  A static array (the only LDS object, so it sits at address 0) lets
     // every tile and slot offset fold into the immediate field of the LDS reads.
-    __shared__ __attribute__((aligned(1024))) char smem[NSLOT * (KTILE + VTILE)];
+    // 16 more bytes at the end carry the next work item's number from thread 0 to the rest of the workgroup.
+    __shared__ __attribute__((aligned(1024))) char smem[NSLOT * (KTILE + VTILE) + 16];
+    constexpr int NEXT_OFF = NSLOT * (KTILE + VTILE);
     constexpr int VOFF = NSLOT * KTILE;
     // The immediate offset of an LDS read reaches 64 KB.  K reads stay below that; V reads go through address
     // registers biased by VBIAS so that VOFF - VBIAS + slot and tile offsets fit the immediate as well.
@@ -103,8 +105,33 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     const int g = lane >> 5;
     const int l32 = lane & 31;
 
+    // Persistent workgroups: the grid holds as many workgroups as the chip keeps resident, and each takes work
+    // items of its XCD (heaviest first) until none is left.  This spares the launch of a workgroup per item
+    // (2-3 us of an idle CU slot each time).  With a queue (one counter per XCD in the caller's workspace, set to
+    // the number of workgroups per XCD before the launch) the next item is whatever the counter hands out, asked
+    // for at the start of the current item so that the answer is there at its end; without one the items are
+    // dealt with a stride, in alternating direction from round to round, so that a workgroup that got the
+    // heaviest item of one round gets the lightest of the next.
+    const int GL = gridDim.x >> 3, lw = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+    const int slots_per_xcd = p_arg.slots_per_xcd;
+    int* const queue = p_arg.queue ? p_arg.queue + xcd * 16 : nullptr;
+    int round = 0;
+    int slot = lw;
+    auto process_item = [&]() __attribute__((always_inline)) {
+    // Per-lane values that depend on the lane number only are recomputed for every item (a few dozen VALU
+    // instructions): hoisted out of the item loop they would be spilled.  The empty asm hides from the compiler
+    // that the lane number is the same every time.
+    int lane_v = lane;
+    asm volatile("" : "+v"(lane_v));
+    // The parameters are read from the kernel argument segment again for every item (scalar loads that hit the
+    // scalar cache): held in registers across the loop, they and everything the compiler derives from them
+    // ahead of the loop would not fit the scalar register file.
+    const __attribute__((address_space(4))) FwdParams* pk =
+        (const __attribute__((address_space(4))) FwdParams*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(pk));
+    const FwdParams& p = *(const FwdParams*)pk;
     Work W;
-    if (!decode_work<BM, BN>(p, W)) return;
+    if (!decode_work<BM, BN>(p, W, slot * 8 + xcd)) return;
     const SeqMask& M = W.M;
     const int n = W.n, nq = W.nq;
 
@@ -144,8 +171,8 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     typedef TileCopy<BN, VROW, true, ES> VCopy;
     KCopy kcopy;
     VCopy vcopy;
-    kcopy.init(wave, lane, k_rsb, n);
-    vcopy.init(wave, lane, v_rsb, n);
+    kcopy.init(wave, lane_v, k_rsb, n);
+    vcopy.init(wave, lane_v, v_rsb, n);
     constexpr int NPW = KCopy::PER_WAVE + VCopy::PER_WAVE;  // copy instructions per wave and step
     static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
 
@@ -168,7 +195,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
 
     int kaddr[KS];
     int vaddr[2][DT];
-    lds_read_offsets<TT, DQK, DV>(kaddr, vaddr, lane);
+    lds_read_offsets<TT, DQK, DV>(kaddr, vaddr, lane_v);
 #pragma unroll
     for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
@@ -374,6 +401,29 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         if (W.split == 0 && threadIdx.x == 0) p.split_counts[W.block_id] = W.nsplit;
     } else
         store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
+    };  // process_item
+    int parity = 0;  // two hand-over words used in turn: a wave may still be reading one when thread 0, an item
+                     // without barriers later, writes the next
+    while (slot < slots_per_xcd) {
+        int ticket = 0;           // per lane; only thread 0's is meaningful
+        int next = 0x7fffffff;    // wave-uniform
+        if (queue) {
+            if (threadIdx.x == 0) ticket = atomicAdd(queue, 1);
+        } else {
+            ++round;
+            if (round * GL < slots_per_xcd) next = round * GL + ((round & 1) ? GL - 1 - lw : lw);
+        }
+        process_item();
+        if (queue) {
+            if (threadIdx.x == 0) *HSTU_LDS(int, smem + NEXT_OFF + parity * 4) = ticket;
+            __syncthreads();  // hands over the ticket, and every wave is done with the LDS tiles of this item
+            next = *HSTU_LDS(const int, smem + NEXT_OFF + parity * 4);
+            parity ^= 1;
+        } else {
+            __syncthreads();  // every wave is done with the LDS tiles before the next item's first copies land
+        }
+        slot = __builtin_amdgcn_readfirstlane(next);
+    }
 }
 
 }  // namespace hstu

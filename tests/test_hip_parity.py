@@ -284,7 +284,31 @@ def test_kv_splits_rejections_and_auto(pkg, dev):
     a.batch, a.heads, a.dqk, a.dv, a.delta_size = 32, 4, 128, 128, 256
     a.total_q, a.total_kv, a.max_seq_len = 32 * 256, 32 * 3000, 4352
     need = hb.lib().hstu_hip_workspace_bytes(ctypes.byref(a))
-    assert need == 4 * 128 + 2 * a.total_q * 4 * 128 * 4 + 256  # run counts, two fp32 partial outputs, alignment slack
+    # work-item counters, run counts, two fp32 partial outputs, alignment slack
+    assert need == 512 + 4 * 128 + 2 * a.total_q * 4 * 128 * 4 + 256
+
+
+@pytest.mark.parametrize("cfg", [2, 3])
+@pytest.mark.parametrize("ragged", [False, True])
+def test_more_work_items_than_resident_workgroups(pkg, dev, cfg, ragged):
+    """Batches with several work items per resident workgroup: equal lengths take the strided deal, ragged ones
+    the per-XCD counters; with targets and a window so that item order cannot hide a mask mistake."""
+    _announce("persistent rounds", cfg, ragged)
+    B, H, D, N = 40, 2, 64, 1536
+    rng = np.random.default_rng(2024)
+    lengths = rng.integers(1, N + 1, size=B) if ragged else np.full(B, N)
+    if ragged:
+        lengths[3] = 0
+        lengths[7] = N
+    tg = np.minimum(rng.integers(0, 40, size=B), lengths)
+    q, k, v, offs, t = make_case(99, lengths, H, D, targets=tg)
+    alpha = 1.0 / D**0.5
+    for w in (0, 500):
+        got = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, 0, 0, cfg)
+        ref = _ref_full(q, k, v, offs, t, N, alpha, w, 0, 0)
+        assert_parity(got, ref, f"w={w}")
+        again = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, 0, 0, cfg)
+        assert torch.equal(got, again), "item order must not change the result"
 
 
 def test_invariants_on_device(pkg, dev):
