@@ -106,17 +106,20 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     const int l32 = lane & 31;
 
     // Persistent workgroups: the grid holds as many workgroups as the chip keeps resident, and each takes work
-    // items of its XCD (heaviest first) until none is left.  This spares the launch of a workgroup per item
-    // (2-3 us of an idle CU slot each time).  With a queue (one counter per XCD in the caller's workspace, set to
-    // the number of workgroups per XCD before the launch) the next item is whatever the counter hands out, asked
-    // for at the start of the current item so that the answer is there at its end; without one the items are
-    // dealt with a stride, in alternating direction from round to round, so that a workgroup that got the
-    // heaviest item of one round gets the lightest of the next.
+    // items (heaviest first) until none is left.  This spares the launch of a workgroup per item (2-3 us of an
+    // idle CU slot each time).  Item ids are slot * 8 + xcd: the items of one XCD's list share K/V through that
+    // XCD's L2.  With a queue (one counter per XCD in the caller's workspace, set to the number of workgroups per
+    // XCD before the launch) the next item is whatever the counter of the workgroup's own XCD hands out, asked for
+    // at the start of the current item so that the answer is there at its end; when that list is exhausted the
+    // workgroup goes on with the lists of the other XCDs (the XCDs do not run equally fast, and a ragged batch
+    // does not split evenly).  Without a queue the items of the own list are dealt with a stride, in alternating
+    // direction from round to round, so that a workgroup that got the heaviest item of one round gets the
+    // lightest of the next.
     const int GL = gridDim.x >> 3, lw = blockIdx.x >> 3, xcd = blockIdx.x & 7;
     const int slots_per_xcd = p_arg.slots_per_xcd;
-    int* const queue = p_arg.queue ? p_arg.queue + xcd * 16 : nullptr;
+    int* const queue = p_arg.queue;
     int round = 0;
-    int slot = lw;
+    int bid = lw < slots_per_xcd ? lw * 8 + xcd : -1;
     auto process_item = [&]() __attribute__((always_inline)) {
     // Per-lane values that depend on the lane number only are recomputed for every item (a few dozen VALU
     // instructions): hoisted out of the item loop they would be spilled.  The empty asm hides from the compiler
@@ -131,7 +134,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     asm volatile("" : "+s"(pk));
     const FwdParams& p = *(const FwdParams*)pk;
     Work W;
-    if (!decode_work<BM, BN>(p, W, slot * 8 + xcd)) return;
+    if (!decode_work<BM, BN>(p, W, bid)) return;
     const SeqMask& M = W.M;
     const int n = W.n, nq = W.nq;
 
@@ -404,25 +407,39 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     };  // process_item
     int parity = 0;  // two hand-over words used in turn: a wave may still be reading one when thread 0, an item
                      // without barriers later, writes the next
-    while (slot < slots_per_xcd) {
-        int ticket = 0;           // per lane; only thread 0's is meaningful
-        int next = 0x7fffffff;    // wave-uniform
+    int victim = xcd;  // whose list thread 0 draws from
+    while (bid >= 0) {
+        int ticket = 0;  // per lane; only thread 0's is meaningful
+        int next = -1;   // wave-uniform
         if (queue) {
-            if (threadIdx.x == 0) ticket = atomicAdd(queue, 1);
+            if (threadIdx.x == 0) ticket = atomicAdd(queue + victim * 16, 1);
         } else {
             ++round;
-            if (round * GL < slots_per_xcd) next = round * GL + ((round & 1) ? GL - 1 - lw : lw);
+            const int ns = round * GL + ((round & 1) ? GL - 1 - lw : lw);
+            if (ns < slots_per_xcd) next = ns * 8 + xcd;
         }
         process_item();
         if (queue) {
-            if (threadIdx.x == 0) *HSTU_LDS(int, smem + NEXT_OFF + parity * 4) = ticket;
-            __syncthreads();  // hands over the ticket, and every wave is done with the LDS tiles of this item
+            if (threadIdx.x == 0) {
+                int nb = -1;
+                for (int tries = 0;;) {
+                    if (ticket < slots_per_xcd) {
+                        nb = ticket * 8 + victim;
+                        break;
+                    }
+                    if (++tries == 8) break;  // every list is exhausted
+                    victim = (victim + 1) & 7;
+                    ticket = atomicAdd(queue + victim * 16, 1);
+                }
+                *HSTU_LDS(int, smem + NEXT_OFF + parity * 4) = nb;
+            }
+            __syncthreads();  // hands over the next item, and every wave is done with the LDS tiles of this one
             next = *HSTU_LDS(const int, smem + NEXT_OFF + parity * 4);
             parity ^= 1;
         } else {
             __syncthreads();  // every wave is done with the LDS tiles before the next item's first copies land
         }
-        slot = __builtin_amdgcn_readfirstlane(next);
+        bid = __builtin_amdgcn_readfirstlane(next);
     }
 }
 
