@@ -501,6 +501,39 @@ __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int
         }
 }
 
+// The same store made row-contiguous: the wave first writes its 32 x DV output tile (16-bit elements) to its own
+// LDS area `lds` (32 rows of DV*2 + 16 bytes; the pad spreads the rows over the banks), then reads it back 16
+// bytes per lane, 16 (or 8, 4) lanes per row, so that one store instruction covers whole rows.  The direct
+// store above touches 32 rows per instruction, 16 bytes in each, which is slow to issue.
+// Only the wave itself touches `lds`; the caller makes sure nobody still reads what was there before.
+template <class TT, int DT>
+__device__ __forceinline__ void store_output_via_lds(const f32x16_t (&oacc)[DT][1], char* lds, char* o, int64_t orow0, int q0,
+                                                     int nq, int64_t o_rs, int64_t o_hs, int h, int lane, float oscale) {
+    typedef typename TT::out_elem elem;  // 16 bits
+    typedef __attribute__((ext_vector_type(4))) elem elem4;
+    constexpr int ROWB = DT * 64 + 16;    // bytes per LDS row
+    constexpr int CHR = DT * 4;           // 16-byte chunks per output row
+    constexpr int RPI = 64 / CHR;         // rows per store instruction
+    const int l32 = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            elem4 o4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o4[i] = (elem)(oacc[dt][0][r4 * 4 + i] * oscale);
+            *HSTU_LDS(elem4, lds + l32 * ROWB + (dt * 32 + r4 * 8 + g * 4) * 2) = o4;
+        }
+    const int chunk = lane % CHR, rsub = lane / CHR;
+    char* op = o + ((orow0 + q0 + rsub) * o_rs + (int64_t)h * o_hs) * 2 + chunk * 16;
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+        const int row = i * RPI + rsub;
+        const i32x4_t v = *HSTU_LDS(const i32x4_t, lds + row * ROWB + chunk * 16);
+        if (q0 + row < nq) *(i32x4_t*)(op + (int64_t)i * RPI * o_rs * 2) = v;
+    }
+}
+
 // Unscaled fp32 accumulators of one block of 32 query rows to partial[split][row][head][dv]; 16 bytes per store.
 template <int DT, int QT>
 __device__ __forceinline__ void store_partial(const f32x16_t (&oacc)[DT][QT], int qt, float* partial, int64_t orow0, int ql,

@@ -402,8 +402,16 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     if (my_partial) {
         store_partial<DT>(oacc, 0, my_partial, orow0, wq0 + l32, nq, p.H, W.h, g);
         if (W.split == 0 && threadIdx.x == 0) p.split_counts[W.block_id] = W.nsplit;
-    } else
+    } else if constexpr ((NG * 4) * 32 * (DT * 64 + 16) <= NSLOT * (KTILE + VTILE)) {
+        // the K/V tiles are dead once every wave is through its last product; each wave then turns its output
+        // tile around in its own piece of that LDS
+        __syncthreads();
+        store_output_via_lds<TT, DT>(oacc, smem + wave * (32 * (DT * 64 + 16)), p.o, orow0, wq0, nq, p.o_rs, p.o_hs, W.h,
+                                     lane, p.oscale);
+    } else {
+        // 8-bit K/V tiles are smaller than the 16-bit output staging would be
         store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
+    }
     };  // process_item
     int parity = 0;  // two hand-over words used in turn: a wave may still be reading one when thread 0, an item
                      // without barriers later, writes the next
