@@ -135,18 +135,19 @@ struct Plan {
     int cfg;               // tile configuration, 1-based
     int splits;            // workgroups per row block along kv (1 = no split)
     int chunk;             // kv tiles per run when split
-    size_t queue_bytes;    // work-item counters of the persistent kernels, at the start of the workspace
+    size_t queue_bytes;    // work-item counters and list lengths of the persistent kernels, at the start of the workspace
+    size_t items_bytes;    // work lists, behind the partial outputs (8 lists of {b * H + h, row block})
     size_t order_bytes;    // sequence ranking, behind the counters
     size_t counts_bytes;   // runs per row block, behind the ranking
     size_t partial_bytes;  // fp32 partial outputs of the runs, 256-byte aligned behind the counts
-    size_t total() const { return queue_bytes + order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0); }
+    size_t total() const { return queue_bytes + order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0) + items_bytes; }
 };
 
 constexpr int kMaxSplits = 8;
 constexpr int kTileRows = 64;  // kv rows per tile of every configuration
 
 Plan make_plan(const HstuFwdArgs* a) {
-    Plan pl = {0, 1, 0, 0, 0, 0, 0};
+    Plan pl = {0, 1, 0, 0, 0, 0, 0, 0};
     // The ping-pong kernel (256-row blocks, one workgroup per CU) wins when the average sequence is long; the
     // one-group pipeline (128-row blocks, two workgroups per CU) wastes less on short or very uneven sequences
     // and in delta mode.
@@ -163,7 +164,7 @@ Plan make_plan(const HstuFwdArgs* a) {
     }
     if (a->sort_by_length && a->batch >= 2 && a->batch <= kMaxSortBatch) pl.order_bytes = (size_t)a->batch * sizeof(int);
     if (pl.cfg < 2 || a->batch <= 0) return pl;
-    pl.queue_bytes = 8 * 64;  // one counter per XCD, 64 bytes apart
+    pl.queue_bytes = 8 * 64 + 64;  // one counter per XCD, 64 bytes apart, then the 8 list lengths
     const int bm = pl.cfg == 2 ? 256 : 128;
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long blocks = (long long)a->batch * a->heads * ((rows_per_pair + bm - 1) / bm);
@@ -180,6 +181,13 @@ Plan make_plan(const HstuFwdArgs* a) {
         if (want > max_tiles / 16) want = max_tiles / 16;
         if (want > kMaxSplits) want = kMaxSplits;
         if (want >= 2) s = (int)want;
+    }
+    // Work lists for ragged batches (equal lengths are dealt arithmetically, a kv-split enumerates its runs
+    // arithmetically too): 8 bytes per possible item; beyond 64 MB the arithmetic enumeration stays.
+    const bool uniform = a->delta_size == 0 && a->total_kv == (int64_t)a->batch * a->max_seq_len;
+    if (s == 1 && !uniform) {
+        const unsigned long long bytes = (unsigned long long)((a->batch * (long long)a->heads + 7) / 8) * (unsigned long long)((rows_per_pair + bm - 1) / bm) * 64ull;
+        if (bytes <= (64ull << 20)) pl.items_bytes = (size_t)bytes + 8;  // 8: room to align the records
     }
     if (s > 1) {
         pl.splits = s;
@@ -373,6 +381,8 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     if (resident < 1) resident = 1;
     const int grid_per_xcd = (int)(slots < resident ? slots : resident);
     if (cfg < 2 || slots <= grid_per_xcd) queue = nullptr;  // every workgroup has exactly one item
+    int* items = nullptr;
+    if (queue && plan.items_bytes > 0 && ws_bytes >= plan.total()) items = (int*)(ws + plan.total() - plan.items_bytes);
     // Equal-length sequences (every one as long as max_seq_len allows): dealing the items with a fixed stride is
     // perfectly balanced and keeps all workgroups of an XCD on the same (sequence, head) pair at the same time,
     // which measures 4-5 % faster than the counter; any other batch needs the counter for balance.
@@ -391,6 +401,19 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     }
     p.order = order;
     p.queue = queue;
+    if (items && queue) {
+        // the lists are 8-byte records behind everything else in the workspace; align them
+        items = (int*)((reinterpret_cast<uintptr_t>(items) + 7) & ~(uintptr_t)7);
+        p.items_cap = (int)slots;
+        hipLaunchKernelGGL(hstu::hstu_plan_kernel, dim3(8), dim3(HSTU_PLAN_THREADS), 0, stream, p, bm, 64, queue + 8 * 16, items);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            set_last_error("plan kernel launch", e);
+            return HSTU_ERR_LAUNCH;
+        }
+        p.items = items;
+        p.nitems = queue + 8 * 16;
+    }
 
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
     if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);

@@ -64,6 +64,12 @@ struct FwdParams {
     int pairs_per_xcd;  // ceil(B*H / 8)
     int slots_per_xcd;  // work items per XCD = pairs_per_xcd * num_mb * kv_splits
     int* queue;         // NULL, or 8 counters 64 bytes apart (one per XCD) handing out work items
+    // NULL, or the work lists built by hstu_plan_kernel: items[xcd * items_cap + i] = {b * H + h, row block},
+    // heaviest class first, nitems[xcd] entries.  Without them item i of an XCD is decoded arithmetically
+    // and may turn out to hold no work (a row block past the end of a short sequence).
+    const int* items;
+    const int* nitems;
+    int items_cap;
     int max_seq_len;
     int delta;          // 0 = full attention
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
@@ -244,6 +250,20 @@ struct Work {
     SeqMask M;
 };
 
+// Tiles [jt_begin, jt_end) of `bn` kv rows that can hold a valid pair for rows R0..R1 (sequence positions) of a
+// sequence with `u` non-target positions.
+__device__ __forceinline__ void kv_tile_range(const SeqMask& M, int u, int R0, int R1, int bn, int& jt_begin, int& jt_end) {
+    const int idr_lo = M.id(R0);
+    const bool ctx_rows = M.c > 0 && idr_lo == 0;
+    int kv_hi = R1 + 1;
+    if (ctx_rows && u > kv_hi) kv_hi = u;
+    if (kv_hi > M.n) kv_hi = M.n;
+    int kv_lo = 0;
+    if (M.w > 0 && M.f == 0 && !ctx_rows && idr_lo - M.w > 0) kv_lo = idr_lo - M.w + M.shift;
+    jt_end = (kv_hi + bn - 1) / bn;
+    jt_begin = kv_lo / bn;
+}
+
 // Decode work item `bid` (the workgroup id in a one-item-per-workgroup launch).  Workgroup ids go round-robin
 // over the 8 XCDs, so ids congruent mod 8 share an L2: all row blocks of one (sequence, head) pair stay on one
 // XCD, heaviest block first.  Returns false if the item holds no work.
@@ -262,7 +282,16 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     // the first row block (its contextual rows see every non-target key) is the heaviest of all and runs
     // many times longer than the others, so the first row blocks of all pairs are launched before anything else.
     int pair_local, mb;
-    if (p.c > 0) {
+    if (p.items) {
+        // {b * H + h, row block} straight from the list
+        if (slot >= HSTU_CONST(int, p.nitems)[xcd]) return false;
+        const i32x2_t rec = HSTU_CONST(i32x2_t, p.items)[(int64_t)xcd * p.items_cap + slot];
+        const int bh = __builtin_amdgcn_readfirstlane(rec[0]);
+        mb = __builtin_amdgcn_readfirstlane(rec[1]);
+        w.b = bh / p.H;
+        w.h = bh - w.b * p.H;
+        pair_local = 0;
+    } else if (p.c > 0) {
         if (slot < p.pairs_per_xcd) {
             pair_local = slot;
             mb = 0;
@@ -275,6 +304,7 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
         pair_local = slot / p.num_mb;
         mb = p.num_mb - 1 - (slot - pair_local * p.num_mb);
     }
+    if (!p.items) {
     const int pair = pair_local * 8 + xcd;
     if (pair >= p.B * p.H) return false;
     const int rseq = pair / p.H;
@@ -285,6 +315,7 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     // them through the constant address space makes these scalar loads (scalar cache, a fraction of the
     // latency of a vector load), which matters because three of them are chained at the start of every workgroup.
     w.b = p.order ? HSTU_CONST(int, p.order)[rseq] : rseq;
+    }
     int64_t seq_start, seq_end;
     if (p.offsets_i64) {
         seq_start = HSTU_CONST(int64_t, p.offsets)[w.b];
@@ -320,15 +351,7 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     const int m1 = (w.m0 + BM < w.nq ? w.m0 + BM : w.nq);
     w.R0 = w.rbase + w.m0;
     w.R1 = w.rbase + m1 - 1;
-    const int idr_lo = M.id(w.R0);
-    const bool ctx_rows = p.c > 0 && idr_lo == 0;
-    int kv_hi = w.R1 + 1;
-    if (ctx_rows && w.u > kv_hi) kv_hi = w.u;
-    if (kv_hi > n) kv_hi = n;
-    int kv_lo = 0;
-    if (p.w > 0 && p.f == 0 && !ctx_rows && idr_lo - p.w > 0) kv_lo = idr_lo - p.w + M.shift;
-    w.jt_end = (kv_hi + BN - 1) / BN;
-    w.jt_begin = kv_lo / BN;
+    kv_tile_range(M, w.u, w.R0, w.R1, BN, w.jt_begin, w.jt_end);
     w.nsplit = 1;
     w.block_id = (w.b * p.H + w.h) * p.num_mb + mb;
     if (p.kv_splits > 1) {
@@ -340,6 +363,150 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     }
     w.skip_scan = p.w > 0 || p.c > 0 || p.targets != nullptr;
     return true;
+}
+
+// Inclusive prefix sum over the 64 lanes of a wave with data-parallel-primitive moves: shifts by 1, 2, 4, 8
+// inside each row of 16 lanes (lanes without a source add 0), then lane 15 of rows 0 and 2 is added to rows 1
+// and 3, then lane 31 to rows 2 and 3.
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+#define HSTU_PLAN_THREADS 1024
+// Builds the work lists of the persistent kernels: one workgroup per XCD walks the (sequence, head) pairs that
+// XCD owns (pair = 8 * i + xcd, sequences taken in `order` if given) and lists every row block that exists,
+// sorted by weight class (floor(log2(kv tiles)), heaviest class first; within a class in pair order, within a
+// pair heaviest block first).  Heavy-first across the whole list keeps the end of the launch made of small
+// items, items of one class and pair stay neighbours (they share K/V through the L2), and row blocks past the
+// end of short sequences never become items.  A stable counting sort: the candidate items in pair-major order
+// are cut into 256 equal runs, one per thread; count per thread and class, scan over the threads, place.
+__global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(const FwdParams p, int bm, int bn, int* nitems, int* items) {
+    constexpr int NC = 12;    // classes: up to 2^11 = 2048 tiles and more
+    constexpr int NT = HSTU_PLAN_THREADS, NW = NT / 64;
+    constexpr int CACHE = 32768;  // candidates whose class is remembered between the two walks
+    __shared__ int cnt[NC][NT];
+    __shared__ int wave_sum[NC][NW];
+    __shared__ int cbase[NC];
+    __shared__ signed char cls[CACHE];  // weight class of candidate k, -1 = no such row block
+    const int xcd = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int c = 0; c < NC; ++c) cnt[c][tid] = 0;
+    const int num_mb = p.num_mb;
+    const int total = p.pairs_per_xcd * num_mb;  // candidates: every row block a pair could have
+    const int run = (total + NT - 1) / NT;
+    const int k_end = (tid + 1) * run < total ? (tid + 1) * run : total;
+    auto walk = [&](bool place) {
+        int cur_pl = -1, bh = 0, n = 0, nq = 0, rbase = 0, u = 0;
+        bool live = false;
+        SeqMask M;
+        for (int k = tid * run; k < k_end; ++k) {
+            const int pl = k / num_mb;
+            const int mb = num_mb - 1 - (k - pl * num_mb);  // heaviest block of a pair first
+            if (place && k < CACHE) {
+                // second walk: the class is known, only the pair's identity has to be looked up again
+                const int c = cls[k];
+                if (c < 0) continue;
+                if (pl != cur_pl) {
+                    cur_pl = pl;
+                    const int pair = pl * 8 + xcd;
+                    const int rseq = pair / p.H;
+                    bh = (p.order ? p.order[rseq] : rseq) * p.H + (pair - rseq * p.H);
+                }
+                const int pos = cbase[c] + cnt[c][tid];
+                if (pos < p.items_cap) {
+                    items[2 * ((int64_t)xcd * p.items_cap + pos)] = bh;
+                    items[2 * ((int64_t)xcd * p.items_cap + pos) + 1] = mb;
+                }
+                cnt[c][tid] += 1;
+                continue;
+            }
+            if (!place && k < CACHE) cls[k] = -1;
+            if (pl != cur_pl) {
+                cur_pl = pl;
+                const int pair = pl * 8 + xcd;
+                live = pair < p.B * p.H;
+                if (live) {
+                    const int rseq = pair / p.H;
+                    const int b = p.order ? p.order[rseq] : rseq;
+                    bh = b * p.H + (pair - rseq * p.H);
+                    const int64_t len = p.offsets_i64 ? ((const int64_t*)p.offsets)[b + 1] - ((const int64_t*)p.offsets)[b]
+                                                      : (int64_t)(((const int*)p.offsets)[b + 1] - ((const int*)p.offsets)[b]);
+                    n = len > p.max_seq_len ? p.max_seq_len : (int)len;
+                    nq = p.delta > 0 ? p.delta : n;
+                    rbase = p.delta > 0 ? n - p.delta : 0;
+                    live = n > 0 && rbase >= 0;
+                    int t = 0;
+                    if (p.targets) t = p.targets_i64 ? (int)((const int64_t*)p.targets)[b] : ((const int*)p.targets)[b];
+                    M.n = n;
+                    M.w = p.w;
+                    M.c = p.c;
+                    M.f = p.f;
+                    M.shift = p.c > 0 ? p.c - 1 : 0;
+                    u = n - t;
+                    M.max_id = u - M.shift;
+                    M.idclamp = p.targets ? M.max_id : 0x7fffffff;
+                }
+            }
+            const int m0 = mb * bm;
+            if (!live || m0 >= nq) continue;
+            const int m1 = m0 + bm < nq ? m0 + bm : nq;
+            int jb, je;
+            kv_tile_range(M, u, rbase + m0, rbase + m1 - 1, bn, jb, je);
+            const int tiles = je - jb;
+            if (tiles <= 0) continue;
+            int c = 31 - __builtin_clz((unsigned)tiles);
+            c = c > NC - 1 ? NC - 1 : c;
+            if (!place && k < CACHE) cls[k] = (signed char)c;
+            if (place) {
+                const int pos = cbase[c] + cnt[c][tid];
+                if (pos < p.items_cap) {
+                    items[2 * ((int64_t)xcd * p.items_cap + pos)] = bh;
+                    items[2 * ((int64_t)xcd * p.items_cap + pos) + 1] = mb;
+                }
+            }
+            cnt[c][tid] += 1;
+        }
+    };
+    walk(false);
+    __syncthreads();
+    // exclusive scan over the threads for every class: within a wave by shuffles, across waves through LDS
+    int excl[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int v = cnt[c][tid];
+        const int incl = wave_inclusive_scan(v);
+        excl[c] = incl - v;
+        if (lane == 63) wave_sum[c][wave] = incl;
+    }
+    __syncthreads();
+    if (tid < NC) {  // per class: wave sums -> exclusive prefix over the waves, and the class total
+        int run_sum = 0;
+        for (int w = 0; w < NW; ++w) {
+            const int x = wave_sum[tid][w];
+            wave_sum[tid][w] = run_sum;
+            run_sum += x;
+        }
+        cbase[tid] = run_sum;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int start = 0;
+        for (int c = NC - 1; c >= 0; --c) {  // heaviest class first
+            const int x = cbase[c];
+            cbase[c] = start;
+            start += x;
+        }
+        nitems[xcd] = start < p.items_cap ? start : p.items_cap;
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) cnt[c][tid] = excl[c] + wave_sum[c][wave];
+    __syncthreads();
+    walk(true);
 }
 
 // First tile index >= jt that holds a valid pair for the workgroup's rows (jt_end if none).

@@ -116,7 +116,8 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     // direction from round to round, so that a workgroup that got the heaviest item of one round gets the
     // lightest of the next.
     const int GL = gridDim.x >> 3, lw = blockIdx.x >> 3, xcd = blockIdx.x & 7;
-    const int slots_per_xcd = p_arg.slots_per_xcd;
+    // with work lists the number of items of an XCD is what the plan kernel counted
+    const int slots_per_xcd = p_arg.nitems ? HSTU_CONST(int, p_arg.nitems)[xcd] : p_arg.slots_per_xcd;
     int* const queue = p_arg.queue;
     int round = 0;
     int bid = lw < slots_per_xcd ? lw * 8 + xcd : -1;
@@ -415,7 +416,8 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     };  // process_item
     int parity = 0;  // two hand-over words used in turn: a wave may still be reading one when thread 0, an item
                      // without barriers later, writes the next
-    int victim = xcd;  // whose list thread 0 draws from
+    int victim = xcd;           // whose list thread 0 draws from ...
+    int limit = slots_per_xcd;  // ... and how many items that list holds
     while (bid >= 0) {
         int ticket = 0;  // per lane; only thread 0's is meaningful
         int next = -1;   // wave-uniform
@@ -431,12 +433,13 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
             if (threadIdx.x == 0) {
                 int nb = -1;
                 for (int tries = 0;;) {
-                    if (ticket < slots_per_xcd) {
+                    if (ticket < limit) {
                         nb = ticket * 8 + victim;
                         break;
                     }
                     if (++tries == 8) break;  // every list is exhausted
                     victim = (victim + 1) & 7;
+                    if (p_arg.nitems) limit = p_arg.nitems[victim];
                     ticket = atomicAdd(queue + victim * 16, 1);
                 }
                 *HSTU_LDS(int, smem + NEXT_OFF + parity * 4) = nb;

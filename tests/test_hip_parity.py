@@ -284,8 +284,8 @@ def test_kv_splits_rejections_and_auto(pkg, dev):
     a.batch, a.heads, a.dqk, a.dv, a.delta_size = 32, 4, 128, 128, 256
     a.total_q, a.total_kv, a.max_seq_len = 32 * 256, 32 * 3000, 4352
     need = hb.lib().hstu_hip_workspace_bytes(ctypes.byref(a))
-    # work-item counters, run counts, two fp32 partial outputs, alignment slack
-    assert need == 512 + 4 * 128 + 2 * a.total_q * 4 * 128 * 4 + 256
+    # work-item counters and list lengths, run counts, two fp32 partial outputs, alignment slack
+    assert need == 576 + 4 * 128 + 2 * a.total_q * 4 * 128 * 4 + 256
 
 
 @pytest.mark.parametrize("cfg", [2, 3])

@@ -91,13 +91,15 @@ def test_check_args_status_codes(backend):
     assert chk(dtype=2, k_row_stride=4 * 128 + 8) == -4
     assert chk(dtype=0, k_row_stride=4 * 128 + 8) == 0
     assert chk(workspace=0x1002, workspace_bytes=64) == -4
-    # workspace: 8 work-item counters 64 bytes apart for the persistent kernels (tile configs 2 and 3), plus one int
-    # per sequence for sort_by_length
+    # workspace of the persistent kernels (tile configs 2 and 3): 8 work-item counters 64 bytes apart and 8 list
+    # lengths (576 bytes); for batches that are not all of length max_seq_len the work lists (64 bytes per possible
+    # item of one XCD, + 8); for sort_by_length one int per sequence
     need = lambda **o: backend.lib().hstu_hip_workspace_bytes(ctypes.byref(_args(backend, **o)))  # noqa: E731
-    assert need() == 512
+    assert need() == 576 + (1 * 1 * 64 + 8)
+    assert need(total_q=128, total_kv=128) == 576  # 2 sequences of exactly max_seq_len = 64
     assert need(tile_config=1) == 0
-    assert need(sort_by_length=1, batch=64) == 512 + 256
-    assert need(sort_by_length=1, batch=1) == 512
+    assert need(sort_by_length=1, batch=64) == 576 + 256 + (32 * 1 * 64 + 8)
+    assert need(sort_by_length=1, batch=1) == 576 + (1 * 1 * 64 + 8)
     assert need(sort_by_length=1, batch=64, tile_config=1) == 256
     for rc in range(-8, 1):
         assert backend.lib().hstu_hip_status_string(rc)
