@@ -181,8 +181,12 @@ def mha_fwd(
     tile_config: int = 0,
     sort_by_length: bool = False,
     kv_splits: int = 0,
+    workspace_bytes: Optional[int] = None,
 ) -> None:
-    """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors."""
+    """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors.
+
+    ``workspace_bytes``: scratch to hand to the library; ``None`` = as much as it asks for.  With less it skips
+    the scheduling options that do not fit (the result is the same)."""
     a = HstuFwdArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
@@ -215,6 +219,8 @@ def mha_fwd(
     a.kv_splits = kv_splits
     workspace = None
     need = lib().hstu_hip_workspace_bytes(ctypes.byref(a))
+    if workspace_bytes is not None:
+        need = min(need, workspace_bytes)
     if need > 0:
         # scratch for the schedule; the caching allocator keeps it alive until the stream has consumed it
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)

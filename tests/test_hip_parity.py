@@ -506,6 +506,30 @@ def test_sort_by_length_changes_only_the_schedule(pkg, dev, cfg):
     assert_parity(a, _ref_full(q, k, v, offs, t, 2304, 0.09, 500, 0), "sorted")
 
 
+@pytest.mark.parametrize("cfg", [2, 3])
+def test_partial_workspace_gives_the_same_result(pkg, dev, cfg):
+    """A C caller may pass less scratch than asked for: no workspace, counters only, counters + ranking, everything.
+    Each level only changes the schedule."""
+    from generative_recommenders_amd.ops import hip_backend as hb
+
+    _announce("partial workspace", cfg)
+    B, H, D, N = 48, 2, 64, 1400
+    rng = np.random.default_rng(77)
+    lengths = rng.integers(0, N + 1, size=B)
+    q, k, v, offs, t = make_case(123, lengths, H, D, targets=np.minimum(lengths, rng.integers(0, 30, size=B)))
+    qd, kd, vd, od, td = q.to(dev), k.to(dev), v.to(dev), offs.to(dev), t.to(dev)
+    outs = []
+    for ws in (0, 576, 576 + 4 * B, None):
+        out = torch.empty_like(vd)
+        hb.mha_fwd(qd, kd, vd, out, od, td, max_seq_len=N, alpha=0.125, delta_size=0, max_attn_len=300,
+                   contextual_seq_len=0, min_full_attn_seq_len=0, tile_config=cfg, sort_by_length=True, workspace_bytes=ws)
+        torch.cuda.synchronize()
+        outs.append(out)
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    assert_parity(outs[0], _ref_full(q, k, v, offs, t, N, 0.125, 300, 0, 0), "no workspace")
+
+
 def _random_case(seed):
     rng = np.random.default_rng(seed)
     B = int(rng.integers(1, 7))
