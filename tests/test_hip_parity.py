@@ -530,6 +530,48 @@ def test_partial_workspace_gives_the_same_result(pkg, dev, cfg):
     assert_parity(outs[0], _ref_full(q, k, v, offs, t, N, 0.125, 300, 0, 0), "no workspace")
 
 
+def test_hip_graph_replays_match_eager(pkg, dev):
+    """Both entry points captured into a HIP graph (prep, plan, forward and reduce kernels; no memset node): every
+    replay, with eager work and synchronisation in between, reproduces the eager result bit for bit."""
+    _announce("hip graph")
+    rng = np.random.default_rng(31)
+    B, H, D, N = 40, 2, 64, 1200
+    lengths = rng.integers(1, N + 1, size=B)
+    q, k, v, offs, t = make_case(321, lengths, H, D, targets=np.minimum(lengths, rng.integers(0, 20, size=B)))
+    qd, kd, vd, od, td = q.to(dev), k.to(dev), v.to(dev), offs.to(dev), t.to(dev)
+    delta = 64
+    dl = rng.integers(0, 3000, size=4) + delta
+    dq_, dk, dv_, doffs, dt_ = make_case(322, dl, 2, 128, targets=[delta] * 4)
+    idx = torch.cat([torch.arange(int(doffs[b + 1]) - delta, int(doffs[b + 1])) for b in range(4)])
+    dqd, dkd, dvd, doffd, dtd = dq_[idx].contiguous().to(dev), dk.to(dev), dv_.to(dev), doffs.to(dev), dt_.to(dev)
+
+    def full():
+        return pkg.hstu_mha(N, 0.125, qd, kd, vd, od, num_targets=td, max_attn_len=400, sort_by_length=True)
+
+    def cached():
+        return pkg.delta_hstu_mha(int(dl.max()), 0.09, dqd, dkd, dvd, doffd, num_targets=dtd, kv_splits=3)
+
+    eager_full, eager_delta = full(), cached()
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        full(), cached()  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        g_full, g_delta = full(), cached()
+    for i in range(4):
+        g_full.zero_()
+        g_delta.zero_()
+        (qd * 1.0).sum().item()  # eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_full, eager_full), f"replay {i}"
+        assert torch.equal(g_delta, eager_delta), f"replay {i}"
+
+
 def _random_case(seed):
     rng = np.random.default_rng(seed)
     B = int(rng.integers(1, 7))
