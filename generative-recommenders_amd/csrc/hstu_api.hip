@@ -6,9 +6,11 @@
 
 #include <cstdio>
 #include <cstring>
+#include <initializer_list>
 
 #include "hstu_fwd_kernel.h"
 #include "hstu_fwd_pp_kernel.h"
+#include "hstu_jagged_kernels.h"
 
 namespace hstu {
 
@@ -418,6 +420,116 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
     if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
     return launch_dim<hstu::Fp8>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
+}
+
+}  // extern "C"
+
+namespace {
+
+// Largest power of two <= 16 that divides every value given (addresses, strides, row size).
+int common_vector_bytes(std::initializer_list<uint64_t> values) {
+    uint64_t all = 16;
+    for (uint64_t v : values) all |= v;
+    int vec = 1;
+    while (vec < 16 && (all & vec) == 0) vec <<= 1;
+    return vec;
+}
+
+constexpr int kJaggedRows = 32;  // joined rows per workgroup
+
+int check_jagged_args(const HstuJaggedCopyArgs* a) {
+    if (!a) return HSTU_ERR_NULL_POINTER;
+    if (a->batch < 0 || a->row_bytes < 0 || a->max_len_left < 0 || a->max_len_right < 0 || a->total_left < 0 || a->total_right < 0)
+        return HSTU_ERR_BAD_SHAPE;
+    if (a->left_row_stride < a->row_bytes || a->right_row_stride < a->row_bytes || a->joined_row_stride < a->row_bytes)
+        return HSTU_ERR_BAD_SHAPE;
+    if (!a->offsets_left && a->total_left != (int64_t)a->batch * a->max_len_left) return HSTU_ERR_BAD_SHAPE;
+    if (!a->offsets_right && a->total_right != (int64_t)a->batch * a->max_len_right) return HSTU_ERR_BAD_SHAPE;
+    if (a->batch == 0 || a->row_bytes == 0 || a->total_left + a->total_right == 0) return HSTU_OK;
+    if (!a->joined || (a->total_left > 0 && !a->left) || (a->total_right > 0 && !a->right)) return HSTU_ERR_NULL_POINTER;
+    return HSTU_OK;
+}
+
+template <bool SPLIT>
+int launch_jagged_copy(const HstuJaggedCopyArgs* a, hipStream_t stream) {
+    g_last_error[0] = 0;
+    int rc = check_jagged_args(a);
+    if (rc != HSTU_OK) return rc;
+    if (a->batch == 0 || a->row_bytes == 0 || a->total_left + a->total_right == 0) return HSTU_OK;
+    hstu::JaggedCopyParams p;
+    p.left = (char*)a->left;
+    p.right = (char*)a->right;
+    p.joined = (char*)a->joined;
+    p.left_rs = a->left_row_stride;
+    p.right_rs = a->right_row_stride;
+    p.joined_rs = a->joined_row_stride;
+    p.row_bytes = a->row_bytes;
+    p.offsets_left = a->offsets_left;
+    p.offsets_right = a->offsets_right;
+    p.offsets_left_i64 = a->offsets_left_i64;
+    p.offsets_right_i64 = a->offsets_right_i64;
+    p.batch = a->batch;
+    p.max_len_left = a->max_len_left;
+    p.max_len_right = a->max_len_right;
+    const long long rows = (long long)a->max_len_left + a->max_len_right;
+    const long long gx = (rows + kJaggedRows - 1) / kJaggedRows;
+    if (gx <= 0) return HSTU_OK;
+    if (gx > 0x7fffffffLL || a->batch > 65535) return HSTU_ERR_BAD_SHAPE;  // grid.y limit
+    const dim3 grid((unsigned)gx, (unsigned)a->batch);
+    const int vec = common_vector_bytes({(uint64_t)(uintptr_t)a->left, (uint64_t)(uintptr_t)a->right, (uint64_t)(uintptr_t)a->joined,
+                                         (uint64_t)a->left_row_stride, (uint64_t)a->right_row_stride,
+                                         (uint64_t)a->joined_row_stride, (uint64_t)a->row_bytes});
+    switch (vec) {
+        case 16: hipLaunchKernelGGL((hstu::hstu_jagged_copy_kernel<SPLIT, 16, kJaggedRows>), grid, dim3(256), 0, stream, p); break;
+        case 8: hipLaunchKernelGGL((hstu::hstu_jagged_copy_kernel<SPLIT, 8, kJaggedRows>), grid, dim3(256), 0, stream, p); break;
+        case 4: hipLaunchKernelGGL((hstu::hstu_jagged_copy_kernel<SPLIT, 4, kJaggedRows>), grid, dim3(256), 0, stream, p); break;
+        case 2: hipLaunchKernelGGL((hstu::hstu_jagged_copy_kernel<SPLIT, 2, kJaggedRows>), grid, dim3(256), 0, stream, p); break;
+        default: hipLaunchKernelGGL((hstu::hstu_jagged_copy_kernel<SPLIT, 1, kJaggedRows>), grid, dim3(256), 0, stream, p); break;
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_last_error("jagged copy kernel launch", e);
+        return HSTU_ERR_LAUNCH;
+    }
+    return HSTU_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hstu_hip_concat_2d_jagged(const HstuJaggedCopyArgs* a, void* stream) { return launch_jagged_copy<false>(a, (hipStream_t)stream); }
+
+int hstu_hip_split_2d_jagged(const HstuJaggedCopyArgs* a, void* stream) { return launch_jagged_copy<true>(a, (hipStream_t)stream); }
+
+int hstu_hip_jagged_write_tail(void* joined, int64_t joined_row_stride, const void* offsets, int32_t offsets_i64, const void* tail,
+                               int64_t tail_row_stride, int64_t row_bytes, int32_t batch, int32_t tail_len, void* stream_) {
+    g_last_error[0] = 0;
+    if (batch < 0 || tail_len < 0 || row_bytes < 0 || joined_row_stride < row_bytes || tail_row_stride < row_bytes) return HSTU_ERR_BAD_SHAPE;
+    if (batch == 0 || tail_len == 0 || row_bytes == 0) return HSTU_OK;
+    if (!joined || !offsets || !tail) return HSTU_ERR_NULL_POINTER;
+    if (batch > 65535) return HSTU_ERR_BAD_SHAPE;
+    const dim3 grid((unsigned)((tail_len + kJaggedRows - 1) / kJaggedRows), (unsigned)batch);
+    hipStream_t stream = (hipStream_t)stream_;
+    const int vec = common_vector_bytes({(uint64_t)(uintptr_t)joined, (uint64_t)(uintptr_t)tail, (uint64_t)joined_row_stride,
+                                         (uint64_t)tail_row_stride, (uint64_t)row_bytes});
+#define HSTU_TAIL_LAUNCH(V)                                                                                                   \
+    hipLaunchKernelGGL((hstu::hstu_jagged_write_tail_kernel<V, kJaggedRows>), grid, dim3(256), 0, stream, (char*)joined,        \
+                       joined_row_stride, offsets, offsets_i64, (const char*)tail, tail_row_stride, row_bytes, tail_len)
+    switch (vec) {
+        case 16: HSTU_TAIL_LAUNCH(16); break;
+        case 8: HSTU_TAIL_LAUNCH(8); break;
+        case 4: HSTU_TAIL_LAUNCH(4); break;
+        case 2: HSTU_TAIL_LAUNCH(2); break;
+        default: HSTU_TAIL_LAUNCH(1); break;
+    }
+#undef HSTU_TAIL_LAUNCH
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_last_error("jagged write-tail kernel launch", e);
+        return HSTU_ERR_LAUNCH;
+    }
+    return HSTU_OK;
 }
 
 }  // extern "C"

@@ -55,6 +55,29 @@ class HstuFwdArgs(ctypes.Structure):
     ]
 
 
+class HstuJaggedCopyArgs(ctypes.Structure):
+    """Mirror of ``HstuJaggedCopyArgs`` in include/hstu_hip.h (field order and types must match)."""
+
+    _fields_ = [
+        ("left", ctypes.c_void_p),
+        ("right", ctypes.c_void_p),
+        ("joined", ctypes.c_void_p),
+        ("left_row_stride", ctypes.c_int64),
+        ("right_row_stride", ctypes.c_int64),
+        ("joined_row_stride", ctypes.c_int64),
+        ("row_bytes", ctypes.c_int64),
+        ("offsets_left", ctypes.c_void_p),
+        ("offsets_right", ctypes.c_void_p),
+        ("offsets_left_i64", ctypes.c_int32),
+        ("offsets_right_i64", ctypes.c_int32),
+        ("batch", ctypes.c_int32),
+        ("max_len_left", ctypes.c_int32),
+        ("max_len_right", ctypes.c_int32),
+        ("total_left", ctypes.c_int64),
+        ("total_right", ctypes.c_int64),
+    ]
+
+
 EXPORTS = (
     "hstu_hip_version",
     "hstu_hip_status_string",
@@ -65,6 +88,9 @@ EXPORTS = (
     "hstu_hip_plan",
     "hstu_hip_tile_configs",
     "hstu_hip_tile_config_name",
+    "hstu_hip_concat_2d_jagged",
+    "hstu_hip_split_2d_jagged",
+    "hstu_hip_jagged_write_tail",
 )
 
 _lib: Optional[ctypes.CDLL] = None
@@ -99,6 +125,15 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_tile_configs.restype = ctypes.c_int
         L.hstu_hip_tile_config_name.restype = ctypes.c_char_p
         L.hstu_hip_tile_config_name.argtypes = [ctypes.c_int]
+        for name in ("hstu_hip_concat_2d_jagged", "hstu_hip_split_2d_jagged"):
+            fn = getattr(L, name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.POINTER(HstuJaggedCopyArgs), ctypes.c_void_p]
+        L.hstu_hip_jagged_write_tail.restype = ctypes.c_int
+        L.hstu_hip_jagged_write_tail.argtypes = [
+            ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p, ctypes.c_int64,
+            ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
+        ]
         _lib = L
     return _lib
 
@@ -229,4 +264,55 @@ def mha_fwd(
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         rc = lib().hstu_hip_mha_fwd(ctypes.byref(a), ctypes.c_void_p(stream))
+    raise_for_status(rc)
+
+
+def _offsets_ptr(offsets: Optional[torch.Tensor]):
+    if offsets is None:
+        return None, 0
+    return offsets.data_ptr(), 1 if offsets.dtype == torch.int64 else 0
+
+
+def jagged_copy(
+    split: bool,
+    left: torch.Tensor,
+    right: torch.Tensor,
+    joined: torch.Tensor,
+    offsets_left: Optional[torch.Tensor],
+    offsets_right: Optional[torch.Tensor],
+    batch: int,
+    max_len_left: int,
+    max_len_right: int,
+) -> None:
+    """``left``, ``right`` -> ``joined`` (``split=False``) or back (``split=True``) on the current stream.
+    2-D device tensors of one dtype and row width, innermost stride 1."""
+    a = HstuJaggedCopyArgs()
+    es = joined.element_size()
+    a.left, a.right, a.joined = left.data_ptr(), right.data_ptr(), joined.data_ptr()
+    a.left_row_stride = (left.stride(0) if left.shape[0] > 1 else left.shape[1]) * es
+    a.right_row_stride = (right.stride(0) if right.shape[0] > 1 else right.shape[1]) * es
+    a.joined_row_stride = (joined.stride(0) if joined.shape[0] > 1 else joined.shape[1]) * es
+    a.row_bytes = joined.shape[1] * es
+    a.offsets_left, a.offsets_left_i64 = _offsets_ptr(offsets_left)
+    a.offsets_right, a.offsets_right_i64 = _offsets_ptr(offsets_right)
+    a.batch = batch
+    a.max_len_left, a.max_len_right = max_len_left, max_len_right
+    a.total_left, a.total_right = left.shape[0], right.shape[0]
+    with torch.cuda.device(joined.device):
+        stream = torch.cuda.current_stream(joined.device).cuda_stream
+        fn = lib().hstu_hip_split_2d_jagged if split else lib().hstu_hip_concat_2d_jagged
+        rc = fn(ctypes.byref(a), ctypes.c_void_p(stream))
+    raise_for_status(rc)
+
+
+def jagged_write_tail(joined: torch.Tensor, offsets: torch.Tensor, tail: torch.Tensor, batch: int, tail_len: int) -> None:
+    """``joined[offsets[b+1] - tail_len + i] = tail[b * tail_len + i]`` in place, on the current stream."""
+    es = joined.element_size()
+    optr, i64 = _offsets_ptr(offsets)
+    with torch.cuda.device(joined.device):
+        stream = torch.cuda.current_stream(joined.device).cuda_stream
+        rc = lib().hstu_hip_jagged_write_tail(
+            joined.data_ptr(), joined.stride(0) * es, optr, i64, tail.data_ptr(), tail.stride(0) * es, joined.shape[1] * es,
+            batch, tail_len, ctypes.c_void_p(stream),
+        )
     raise_for_status(rc)

@@ -129,6 +129,50 @@ int hstu_hip_plan(const HstuFwdArgs* args, int32_t* tile_config, int32_t* kv_spl
 int hstu_hip_tile_configs(void);
 const char* hstu_hip_tile_config_name(int id);
 
+/*
+ * ---- The data format either side of the path: per-batch concatenation of two jagged 2-D tensors ----
+ *
+ * `left`, `right` and `joined` are row-major [rows, row_bytes] byte matrices with row strides in BYTES; batch b owns
+ * rows offsets[b] .. offsets[b+1] of a side, or exactly max_len rows when that side's offsets pointer is NULL
+ * ("dense"); `joined` holds, for every batch, the left rows followed by the right rows, batch b starting at row
+ * offsets_left[b] + offsets_right[b].  Caller contract as in the reference: per-batch lengths do not exceed
+ * max_len_left / max_len_right (beyond that the reference's own result is ill-defined -- its mask then selects padding
+ * rows -- and this library leaves the joined rows past max_len_left + max_len_right unwritten).
+ * Replaces `concat_2D_jagged` / `split_2D_jagged` (generative_recommenders/ops/jagged_tensors.py:55-111; semantics
+ * ops/pytorch/pt_jagged_tensors.py:31-173), which the reference uses to build cache (+) delta K/V for
+ * `delta_hstu_mha` and to cut the cache out again (modules/stu.py:84-173).
+ */
+typedef struct HstuJaggedCopyArgs {
+    void* left;                /* [total_left, row_bytes]   input of concat, output of split */
+    void* right;               /* [total_right, row_bytes] */
+    void* joined;              /* [total_left + total_right, row_bytes]   output of concat, input of split */
+    int64_t left_row_stride, right_row_stride, joined_row_stride;  /* bytes, >= row_bytes */
+    int64_t row_bytes;
+    const void* offsets_left;  /* [B+1] or NULL */
+    const void* offsets_right; /* [B+1] or NULL */
+    int32_t offsets_left_i64, offsets_right_i64;  /* 1: int64 elements, 0: int32 */
+    int32_t batch;
+    int32_t max_len_left, max_len_right;
+    int64_t total_left, total_right;  /* rows of `left` and `right` (for validation only) */
+} HstuJaggedCopyArgs;
+
+/* left, right -> joined.  Asynchronous on `stream`; allocates nothing. */
+int hstu_hip_concat_2d_jagged(const HstuJaggedCopyArgs* args, void* stream);
+/* joined -> left, right. */
+int hstu_hip_split_2d_jagged(const HstuJaggedCopyArgs* args, void* stream);
+
+/*
+ * In-place form of the cache (+) delta concatenation: joined[offsets[b+1] - tail_len + i] = tail[b * tail_len + i]
+ * for i < tail_len.  A K/V cache kept as "history rows, then tail_len spare rows" per sequence, with
+ * offsets = kv_caching_offsets + tail_len * arange(B+1) (exactly the offsets `_construct_full_kv` returns,
+ * modules/stu.py:133-173), then needs only the new rows copied per call instead of the whole history.  The
+ * reference has no such entry point; it re-concatenates.  Strides in bytes; every sequence must hold at least
+ * tail_len rows (shorter ones are left untouched).
+ */
+int hstu_hip_jagged_write_tail(void* joined, int64_t joined_row_stride, const void* offsets, int32_t offsets_i64,
+                               const void* tail, int64_t tail_row_stride, int64_t row_bytes, int32_t batch,
+                               int32_t tail_len, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -37,10 +37,11 @@ def test_library_exports_every_declared_symbol(backend):
     assert backend.tile_config_names() == ["m128n64w4", "m256n64w8pp", "m128n64w4pl"]
 
 
-def test_struct_mirror_has_the_header_fields_in_order(backend):
+@pytest.mark.parametrize("struct", ["HstuFwdArgs", "HstuJaggedCopyArgs"])
+def test_struct_mirror_has_the_header_fields_in_order(backend, struct):
     header = open(os.path.join(ROOT, "include", "hstu_hip.h")).read()
-    body = header[header.index("typedef struct HstuFwdArgs {") : header.index("} HstuFwdArgs;")]
-    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S).replace("typedef struct HstuFwdArgs {", "")
+    body = header[header.index(f"typedef struct {struct} {{") : header.index(f"}} {struct};")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S).replace(f"typedef struct {struct} {{", "")
     names = []
     for decl in body.split(";"):
         decl = decl.strip()
@@ -49,7 +50,28 @@ def test_struct_mirror_has_the_header_fields_in_order(backend):
         parts = decl.split(",")
         names.append(re.findall(r"(\w+)\s*$", parts[0].strip())[0])
         names += [p.strip() for p in parts[1:]]
-    assert names == [f[0] for f in backend.HstuFwdArgs._fields_]
+    assert names == [f[0] for f in getattr(backend, struct)._fields_]
+
+
+def test_jagged_copy_argument_checks(backend):
+    """Validation of the jagged copy entry points runs before anything touches the device."""
+    a = backend.HstuJaggedCopyArgs()
+    L = backend.lib()
+    assert L.hstu_hip_concat_2d_jagged(None, None) == -1
+    a.batch, a.row_bytes, a.max_len_left, a.max_len_right = 2, 64, 4, 4
+    a.left_row_stride = a.right_row_stride = a.joined_row_stride = 64
+    a.total_left, a.total_right = 8, 7  # both sides dense: totals must be batch * max_len
+    assert L.hstu_hip_concat_2d_jagged(ctypes.byref(a), None) == -5
+    a.total_right = 8
+    assert L.hstu_hip_concat_2d_jagged(ctypes.byref(a), None) == -1  # pointers missing
+    a.joined_row_stride = 32  # narrower than a row
+    assert L.hstu_hip_split_2d_jagged(ctypes.byref(a), None) == -5
+    a.total_left = a.total_right = a.max_len_left = a.max_len_right = 0
+    a.joined_row_stride = 64
+    assert L.hstu_hip_concat_2d_jagged(ctypes.byref(a), None) == 0  # nothing to copy
+    assert L.hstu_hip_jagged_write_tail(None, 64, None, 1, None, 64, 64, 3, 0, None) == 0
+    assert L.hstu_hip_jagged_write_tail(None, 64, None, 1, None, 64, 64, 3, 2, None) == -1
+    assert L.hstu_hip_jagged_write_tail(None, 32, None, 1, None, 64, 64, 3, 2, None) == -5
 
 
 def _args(backend, **over):
