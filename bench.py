@@ -24,7 +24,8 @@ PEAK_HBM_GBS = 8000.0
 HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced against HBM bandwidth
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"headline": 2.411e9, "cfg2": 0.857e9, "cfg3": 1.362e9, "cfg4": 0.249e9, "cfg5": 2.323e9}
+MEASURED_TRAFFIC_BYTES = {"headline": 2.411e9, "cfg2": 0.857e9, "cfg3": 1.362e9, "cfg4": 0.249e9, "cfg5": 2.323e9,
+                          "kvcat": 0.173e9, "kvtail": 0.0168e9}
 
 
 def run_gpu(wl, args, pkg, workloads, torch):
@@ -109,6 +110,73 @@ def run_cpu_baseline(wl, torch, workloads, budget_s=20.0):
     }
 
 
+def run_jagged(name, args, pkg, torch):
+    """K/V-cache plumbing around delta_hstu_mha at the sizes of cfg4 (32 users, history 1024..4096, 256 new rows, rows of
+    H*D = 512 bf16): `kvcat` = concat_2D_jagged(cache, delta) as the reference's _construct_full_kv does per layer and
+    micro-batch; `kvtail` = write_kv_tail, the in-place form that copies the new rows only."""
+    import numpy as np
+
+    from oracle import jagged_oracle
+
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(1004)
+    B, delta, width = 32, 256, 512
+    hist = rng.integers(1024, 4097, size=B)
+    oc = torch.tensor(np.concatenate([[0], np.cumsum(hist)]), dtype=torch.int64)
+    g = torch.Generator().manual_seed(1004)
+    cache = (torch.randn((int(oc[-1]), width), generator=g) * 0.1).to(torch.bfloat16)
+    new = (torch.randn((B * delta, width), generator=g) * 0.1).to(torch.bfloat16)
+    cache_d, new_d, oc_d = cache.to(dev), new.to(dev), oc.to(dev)
+    full_offsets = (oc + delta * torch.arange(B + 1)).to(dev)
+    max_hist = int(hist.max())
+    full = pkg.concat_2D_jagged(max_hist + delta, cache_d, new_d, max_hist, delta, oc_d, None)
+    if name == "kvcat":
+        def step():
+            return pkg.concat_2D_jagged(max_hist + delta, cache_d, new_d, max_hist, delta, oc_d, None)
+        nbytes = 2 * (cache.numel() + new.numel()) * 2
+        kernel = "hstu_jagged_copy_kernel"
+    else:
+        def step():
+            return pkg.write_kv_tail(full, full_offsets, new_d)
+        nbytes = 2 * new.numel() * 2
+        kernel = "hstu_jagged_write_tail_kernel"
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = start.elapsed_time(stop) / args.steps
+    gbs = nbytes / (ev_ms * 1e-3) / 1e9
+    line = {
+        "metric": "K/V cache (+) delta rows per call, GB/s moved (cfg4 sizes)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": name, "batch": B, "delta_size": delta, "row_bytes": width * 2, "history_rows": int(oc[-1])},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel,
+                     "kernel_ms": round(ev_ms, 4), "algorithmic_bytes": nbytes},
+    }
+    if not args.no_cpu:
+        torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
+        reps, t_used = 0, 0.0
+        dense_off = delta * torch.arange(B + 1)
+        while t_used < 5.0:
+            t0 = time.perf_counter()
+            jagged_oracle.concat_by_batch(cache, new, oc, dense_off)
+            t_used += time.perf_counter() - t0
+            reps += 1
+        cat_bytes = 2 * (cache.numel() + new.numel()) * 2
+        line["cpu_baseline"] = {"value": round(cat_bytes * reps / t_used / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+                                "kind": "port", "sample": f"{reps} full concatenations of the same cache and rows (per-batch torch.cat), {t_used:.1f} s"}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,8 +203,9 @@ def main():
     pkg = __graft_entry__.load_package()
     from generative_recommenders_amd import workloads
 
-    wl = workloads.make_workload(args.workload)
-    if wl.dtype == "fp32":
+    jagged = args.workload in ("kvcat", "kvtail")
+    wl = None if jagged else workloads.make_workload(args.workload)
+    if wl is not None and wl.dtype == "fp32":
         print("bench.py: cfg1 is the CPU correctness case, not a GPU bench workload", file=sys.stderr)
         sys.exit(2)
     if args.calibrate_copy:
@@ -146,6 +215,9 @@ def main():
             dst.copy_(src)  # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
+    if jagged:
+        run_jagged(args.workload, args, pkg, torch)
+        return
     wall_ms, ev_ms = run_gpu(wl, args, pkg, workloads, torch)
     flops = workloads.algorithmic_flops(wl)
     ref_flops = workloads.reference_convention_flops(wl)
