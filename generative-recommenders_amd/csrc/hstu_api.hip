@@ -70,7 +70,8 @@ constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 // `p` arrives complete (num_mb, pairs_per_xcd, slots_per_xcd, queue ...); these only pick the instantiation.
 template <class TT, int DQK, int DV, int QT, int NW, int BN, int OCC>
 int launch(const hstu::FwdParams& p, hipStream_t stream) {
-    constexpr int smem = 2 * BN * (DQK + DV) * TT::ES;
+    // + 64: with dv = 16 the transposing reads of the unused upper half of the tile reach past the last V row
+    constexpr int smem = 2 * BN * (DQK + DV) * TT::ES + 64;
     auto kern = hstu::hstu_fwd_kernel<TT, DQK, DV, QT, NW, BN, OCC>;
     static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; racing threads set the same value
     if (!attr_done) {
@@ -122,8 +123,36 @@ int launch_cfg(const hstu::FwdParams& p, int cfg, int grid_per_xcd, int64_t tota
     return launch<TT, D, D, 1, 4, 64, 2>(p, stream);
 }
 
+// Unequal or 16-wide head dims: only the barrier-per-tile kernel is generic in (dqk, dv).
+template <class TT, int DQK>
+int launch_mixed_dv(const hstu::FwdParams& p, int dv, hipStream_t stream) {
+    switch (dv) {
+        case 16:
+            if constexpr (TT::ES == 2) return launch<TT, DQK, 16, 1, 4, 64, 2>(p, stream);
+            return HSTU_ERR_BAD_HEAD_DIM;
+        case 32: return launch<TT, DQK, 32, 1, 4, 64, 2>(p, stream);
+        case 64: return launch<TT, DQK, 64, 1, 4, 64, 2>(p, stream);
+        case 128: return launch<TT, DQK, 128, 1, 4, 64, 2>(p, stream);
+        default: return HSTU_ERR_BAD_HEAD_DIM;
+    }
+}
+
 template <class TT>
-int launch_dim(const hstu::FwdParams& p, int d, int cfg, int grid_per_xcd, int64_t total_q, hipStream_t stream) {
+int launch_mixed(const hstu::FwdParams& p, int dqk, int dv, hipStream_t stream) {
+    switch (dqk) {
+        case 16:
+            if constexpr (TT::ES == 2) return launch_mixed_dv<TT, 16>(p, dv, stream);
+            return HSTU_ERR_BAD_HEAD_DIM;
+        case 32: return launch_mixed_dv<TT, 32>(p, dv, stream);
+        case 64: return launch_mixed_dv<TT, 64>(p, dv, stream);
+        case 128: return launch_mixed_dv<TT, 128>(p, dv, stream);
+        default: return HSTU_ERR_BAD_HEAD_DIM;
+    }
+}
+
+template <class TT>
+int launch_dim(const hstu::FwdParams& p, int d, int dv, int cfg, int grid_per_xcd, int64_t total_q, hipStream_t stream) {
+    if (cfg == 1 && (d != dv || d == 16)) return launch_mixed<TT>(p, d, dv, stream);
     switch (d) {
         case 32: return launch_cfg<TT, 32>(p, cfg, grid_per_xcd, total_q, stream);
         case 64: return launch_cfg<TT, 64>(p, cfg, grid_per_xcd, total_q, stream);
@@ -155,6 +184,7 @@ Plan make_plan(const HstuFwdArgs* a) {
     // and in delta mode.
     pl.cfg = a->tile_config;
     const long long avg_tiles = a->batch > 0 ? a->total_kv / a->batch / kTileRows : 0;
+    if (a->dqk != a->dv || a->dqk == 16) pl.cfg = 1;  // the only kernel generic in (dqk, dv)
     if (pl.cfg == 0) {
         if (a->delta_size == 0) {
             pl.cfg = avg_tiles >= 3072 / kTileRows ? 2 : 3;
@@ -241,7 +271,7 @@ const char* hstu_hip_status_string(int status) {
         case HSTU_OK: return "ok";
         case HSTU_ERR_NULL_POINTER: return "a required pointer is NULL";
         case HSTU_ERR_BAD_DTYPE: return "only bf16, fp16 and fp8_e4m3 data types are supported";
-        case HSTU_ERR_BAD_HEAD_DIM: return "unsupported head dimension (built: dqk == dv in {32, 64, 128})";
+        case HSTU_ERR_BAD_HEAD_DIM: return "unsupported head dimension (built: dqk, dv in {16, 32, 64, 128}; 8-bit types from 32)";
         case HSTU_ERR_MISALIGNED:
             return "q/k/v/out must be 16-byte aligned with row and head strides that are multiples of 16 bytes";
         case HSTU_ERR_BAD_SHAPE: return "inconsistent sizes";
@@ -288,8 +318,13 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     if (a->tile_config < 0 || a->tile_config > kNumConfigs) return HSTU_ERR_BAD_SHAPE;
     if (a->kv_splits < 0 || a->kv_splits > kMaxSplits || (a->kv_splits > 1 && a->tile_config == 1)) return HSTU_ERR_BAD_SHAPE;
     if (a->workspace && (a->workspace_bytes < 0 || (reinterpret_cast<uintptr_t>(a->workspace) & 3) != 0)) return HSTU_ERR_MISALIGNED;
-    if (a->dqk != a->dv) return HSTU_ERR_BAD_HEAD_DIM;  // as the reference's native op, flash_common.cpp:543-545
-    if (a->dqk != 32 && a->dqk != 64 && a->dqk != 128) return HSTU_ERR_BAD_HEAD_DIM;
+    // head dims 16 / 32 / 64 / 128, independently for q/k and v (the grid of the reference's tests,
+    // hstu_attention_test.py:266-267; its native op wants them equal, flash_common.cpp:543-545); 8-bit rows are at
+    // least 32 wide
+    for (int d : {a->dqk, a->dv})
+        if (d != 32 && d != 64 && d != 128 && !(d == 16 && a->dtype != HSTU_FP8_E4M3)) return HSTU_ERR_BAD_HEAD_DIM;
+    // unequal or 16-wide dims run on tile config 1 only
+    if ((a->dqk != a->dv || a->dqk == 16) && a->tile_config > 1) return HSTU_ERR_UNSUPPORTED;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;  // nothing to do; pointers may be anything
     if (!a->q || !a->k || !a->v || !a->out || !a->seq_offsets) return HSTU_ERR_NULL_POINTER;
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out)) return HSTU_ERR_MISALIGNED;
@@ -417,9 +452,9 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
         p.nitems = queue + 8 * 16;
     }
 
-    if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
-    if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
-    return launch_dim<hstu::Fp8>(p, a->dqk, cfg, grid_per_xcd, a->total_q, stream);
+    if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
+    if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
+    return launch_dim<hstu::Fp8>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
 }
 
 }  // extern "C"

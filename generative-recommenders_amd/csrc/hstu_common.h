@@ -213,6 +213,7 @@ __device__ __forceinline__ int swz_v(int row) {
         if (CH == 8) return (((row >> 1) & 1) | (((row >> 3) & 1) << 1)) << 1;
         return 0;
     }
+    if (CH == 2) return 0;  // 32-byte rows (dv = 16): two chunks, nothing to spread
     const int half_swap = ((row >> 2) & 1) << 1;
     if (CH == 16) return ((row & 3) << 2) | half_swap;
     if (CH == 8) return (((row >> 1) & 1) << 2) | half_swap;
@@ -597,9 +598,10 @@ __device__ __forceinline__ void load_q_operand(typename TT::vec8 (&qreg)[KS], co
 // {8+4g..8+4g+3} (second read), g = l/32 -- the order in which the accumulator of the first product
 // holds its kv rows.
 template <class TT, int DQK, int DV>
-__device__ __forceinline__ void lds_read_offsets(int (&kaddr)[DQK / 16], int (&vaddr)[2][DV / 32], int lane) {
+__device__ __forceinline__ void lds_read_offsets(int (&kaddr)[DQK / 16], int (&vaddr)[2][(DV + 31) / 32], int lane) {
     constexpr int ES = TT::ES;
-    constexpr int KS = DQK / 16, DT = DV / 32, KROW = DQK * ES, VROW = DV * ES, KCH = KROW / 16, VCH = VROW / 16;
+    // DV = 16 still takes one 32-row MFMA: its upper 16 dv rows read whatever follows the row in LDS and are never stored
+    constexpr int KS = DQK / 16, DT = (DV + 31) / 32, KROW = DQK * ES, VROW = DV * ES, KCH = KROW / 16, VCH = VROW / 16;
     const int g = lane >> 5, l32 = lane & 31;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -652,7 +654,8 @@ __device__ __forceinline__ typename TT::vec8 read_vt_operand(const char* lo_addr
 // (dv tile, r/4), stored as 8 bytes.  QT is deduced from the accumulator array.
 template <class TT, int DT, int QT>
 __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int qt, char* o, int64_t orow0, int ql, int nq,
-                                             int64_t o_rs, int64_t o_hs, int h, int g, float oscale) {
+                                             int64_t o_rs, int64_t o_hs, int h, int g, float oscale,
+                                             int dv_valid = 1 << 30) {
     typedef typename TT::out_elem elem;  // 16 bits
     typedef __attribute__((ext_vector_type(4))) elem elem4;
     if (ql >= nq) return;
@@ -661,6 +664,7 @@ __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
+            if (dt * 32 + r4 * 8 >= dv_valid) continue;  // dv = 16: the upper half of the tile does not exist
             elem4 o4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) o4[i] = (elem)(oacc[dt][qt][r4 * 4 + i] * oscale);

@@ -11,11 +11,11 @@ namespace hstu {
 // `sp0` is the sequence position of this lane's first kv slot: tile start + 4*(lane/32).
 template <class TT, int DQK, int DV, int QT, int BN, int MASKED>
 __device__ __forceinline__ void tile_compute(const char* kt, const char* vt, const typename TT::vec8 (&qreg)[QT][DQK / 16],
-                                             f32x16_t (&oacc)[DV / 32][QT], const int (&kaddr)[DQK / 16],
-                                             const int (&vaddr)[2][DV / 32], float c1, const SeqMask& M, int sp0,
+                                             f32x16_t (&oacc)[(DV + 31) / 32][QT], const int (&kaddr)[DQK / 16],
+                                             const int (&vaddr)[2][(DV + 31) / 32], float c1, const SeqMask& M, int sp0,
                                              const RowMask (&rows)[QT]) {
     typedef typename TT::vec8 vec8;
-    constexpr int NS = BN / 32, KS = DQK / 16, DT = DV / 32, KROW = DQK * TT::ES, VROW = DV * TT::ES;
+    constexpr int NS = BN / 32, KS = DQK / 16, DT = (DV + 31) / 32, KROW = DQK * TT::ES, VROW = DV * TT::ES;
     // ---- S^T = K Q^T
     f32x16_t s[NS][QT];
 #pragma unroll
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     typedef typename TT::vec8 vec8;
     constexpr int BM = NW * QT * 32;
     constexpr int KS = DQK / 16;
-    constexpr int DT = DV / 32;
+    constexpr int DT = (DV + 31) / 32;  // dv = 16 computes a 32-row tile and stores half of it
     constexpr int ES = TT::ES;
     constexpr int KROW = DQK * ES, VROW = DV * ES;
     constexpr int KTILE = BN * KROW, VTILE = BN * VROW, STAGE = KTILE + VTILE;
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
 
     const int64_t orow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) store_output<TT, DT>(oacc, qt, p.o, orow0, wq0 + qt * 32 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
+    for (int qt = 0; qt < QT; ++qt) store_output<TT, DT>(oacc, qt, p.o, orow0, wq0 + qt * 32 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale, DV);
 }
 
 }  // namespace hstu

@@ -311,6 +311,33 @@ def test_more_work_items_than_resident_workgroups(pkg, dev, cfg, ragged):
         assert torch.equal(got, again), "item order must not change the result"
 
 
+@pytest.mark.parametrize("dqk,dv", [(16, 16), (16, 128), (128, 16), (32, 64), (64, 32), (128, 64), (64, 128), (32, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_unequal_and_narrow_head_dims(pkg, dev, dqk, dv, dtype):
+    """attn_dim and hidden_dim drawn independently from {16, 32, 64, 128}, as the reference's own test does
+    (hstu_attention_test.py:266-267); full and delta form, with targets, window and contextual prefix."""
+    _announce("mixed dims", dqk, dv, dtype)
+    lengths = [300, 0, 64, 129, 17]
+    q, k, v, offs, t = make_case(1000 + dqk + dv, lengths, 2, dqk, dv, targets=[20, 0, 3, 0, 5], dtype=dtype)
+    if dtype == torch.float16:
+        v.mul_(1024.0)
+    N, alpha = 300, 1.0 / dqk**0.5
+    for w, c in [(0, 0), (50, 4)]:
+        got = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, c, 0, 0)
+        assert got.shape == (sum(lengths), 2, dv)
+        assert_parity(got, _ref_full(q, k, v, offs, t, N, alpha, w, c, 0), f"w={w} c={c}")
+    delta = 16
+    lengths = np.array([200, 16, 77, 130])
+    q, k, v, offs, t = make_case(2000 + dqk + dv, lengths, 2, dqk, dv, targets=[delta] * 4, dtype=dtype)
+    if dtype == torch.float16:
+        v.mul_(1024.0)
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(4)])
+    dq = q[idx].contiguous()
+    got = pkg.delta_hstu_mha(200, alpha, dq.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev))
+    torch.cuda.synchronize()
+    assert_parity(got, O.cached_hstu_mha_per_sequence(200, alpha, dq.float(), k.float(), v.float(), offs, t), "delta")
+
+
 def test_invariants_on_device(pkg, dev):
     """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
     permuting two targets permutes the outputs (stu_test.py:180-321)."""

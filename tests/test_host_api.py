@@ -99,7 +99,10 @@ def test_check_args_status_codes(backend):
     assert chk(seq_offsets=None) == -1
     assert chk(dtype=7) == -2
     assert chk(dqk=48, dv=48) == -3
-    assert chk(dqk=64, dv=128) == -3
+    assert chk(dqk=64, dv=128) == 0  # unequal dims run on tile config 1 ...
+    assert chk(dqk=64, dv=128, tile_config=2) == -6  # ... only
+    assert chk(dqk=16, dv=16, v_row_stride=4 * 16, v_head_stride=16) == 0
+    assert chk(dqk=16, dv=16, dtype=2) == -3  # 8-bit rows are at least 32 wide
     assert chk(q=0x1008) == -4
     assert chk(k_row_stride=4 * 128 + 4) == -4
     assert chk(max_seq_len=0) == -5
