@@ -171,20 +171,27 @@ struct Plan {
     size_t order_bytes;    // sequence ranking, behind the counters
     size_t counts_bytes;   // runs per row block, behind the ranking
     size_t partial_bytes;  // fp32 partial outputs of the runs, 256-byte aligned behind the counts
-    size_t total() const { return queue_bytes + order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0) + items_bytes; }
+    size_t cast_bytes;     // fp16 copies of fp32 q, k, v, each 256-byte aligned, at the very end
+    size_t total() const {
+        return queue_bytes + order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0) + items_bytes + cast_bytes;
+    }
 };
 
 constexpr int kMaxSplits = 8;
 constexpr int kTileRows = 64;  // kv rows per tile of every configuration
 
 Plan make_plan(const HstuFwdArgs* a) {
-    Plan pl = {0, 1, 0, 0, 0, 0, 0, 0};
+    Plan pl = {0, 1, 0, 0, 0, 0, 0, 0, 0};
     // The ping-pong kernel (256-row blocks, one workgroup per CU) wins when the average sequence is long; the
     // one-group pipeline (128-row blocks, two workgroups per CU) wastes less on short or very uneven sequences
     // and in delta mode.
     pl.cfg = a->tile_config;
     const long long avg_tiles = a->batch > 0 ? a->total_kv / a->batch / kTileRows : 0;
     if (a->dqk != a->dv || a->dqk == 16) pl.cfg = 1;  // the only kernel generic in (dqk, dv)
+    if (a->dtype == HSTU_FP32) {
+        pl.cfg = 1;  // and the only one with an fp32 store
+        pl.cast_bytes = 2 * ((size_t)a->total_q * a->heads * a->dqk + (size_t)a->total_kv * a->heads * (a->dqk + a->dv)) + 4 * 256;
+    }
     if (pl.cfg == 0) {
         if (a->delta_size == 0) {
             pl.cfg = avg_tiles >= 3072 / kTileRows ? 2 : 3;
@@ -270,7 +277,7 @@ const char* hstu_hip_status_string(int status) {
     switch (status) {
         case HSTU_OK: return "ok";
         case HSTU_ERR_NULL_POINTER: return "a required pointer is NULL";
-        case HSTU_ERR_BAD_DTYPE: return "only bf16, fp16 and fp8_e4m3 data types are supported";
+        case HSTU_ERR_BAD_DTYPE: return "only bf16, fp16, fp8_e4m3 and fp32 data types are supported";
         case HSTU_ERR_BAD_HEAD_DIM: return "unsupported head dimension (built: dqk, dv in {16, 32, 64, 128}; 8-bit types from 32)";
         case HSTU_ERR_MISALIGNED:
             return "q/k/v/out must be 16-byte aligned with row and head strides that are multiples of 16 bytes";
@@ -308,7 +315,7 @@ const char* hstu_hip_tile_config_name(int id) {
 
 int hstu_hip_check_args(const HstuFwdArgs* a) {
     if (!a) return HSTU_ERR_NULL_POINTER;
-    if (a->dtype != HSTU_BF16 && a->dtype != HSTU_FP16 && a->dtype != HSTU_FP8_E4M3) return HSTU_ERR_BAD_DTYPE;
+    if (a->dtype != HSTU_BF16 && a->dtype != HSTU_FP16 && a->dtype != HSTU_FP8_E4M3 && a->dtype != HSTU_FP32) return HSTU_ERR_BAD_DTYPE;
     if (a->batch < 0 || a->heads <= 0 || a->total_q < 0 || a->total_kv < 0 || a->max_seq_len <= 0 ||
         a->delta_size < 0 || a->max_attn_len < 0 || a->contextual_seq_len < 0 || a->min_full_attn_seq_len < 0)
         return HSTU_ERR_BAD_SHAPE;
@@ -323,17 +330,19 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     // least 32 wide
     for (int d : {a->dqk, a->dv})
         if (d != 32 && d != 64 && d != 128 && !(d == 16 && a->dtype != HSTU_FP8_E4M3)) return HSTU_ERR_BAD_HEAD_DIM;
-    // unequal or 16-wide dims run on tile config 1 only
-    if ((a->dqk != a->dv || a->dqk == 16) && a->tile_config > 1) return HSTU_ERR_UNSUPPORTED;
+    // unequal or 16-wide dims and fp32 run on tile config 1 only
+    if ((a->dqk != a->dv || a->dqk == 16 || a->dtype == HSTU_FP32) && a->tile_config > 1) return HSTU_ERR_UNSUPPORTED;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;  // nothing to do; pointers may be anything
     if (!a->q || !a->k || !a->v || !a->out || !a->seq_offsets) return HSTU_ERR_NULL_POINTER;
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out)) return HSTU_ERR_MISALIGNED;
     const int64_t strides[8] = {a->q_row_stride, a->q_head_stride, a->k_row_stride, a->k_head_stride,
                                 a->v_row_stride, a->v_head_stride, a->o_row_stride, a->o_head_stride};
-    // rows of q/k/v start on 16-byte boundaries: 8 elements of 16 bits, 16 of 8 bits; the output is always 16 bit
-    const int64_t in_mask = a->dtype == HSTU_FP8_E4M3 ? 15 : 7;
+    // rows of q/k/v start on 16-byte boundaries: 8 elements of 16 bits, 16 of 8 bits, 4 of 32 bits; the output is 16
+    // bit, or 32 bit for fp32 inputs
+    const int64_t in_mask = a->dtype == HSTU_FP8_E4M3 ? 15 : a->dtype == HSTU_FP32 ? 3 : 7;
+    const int64_t out_mask = a->dtype == HSTU_FP32 ? 3 : 7;
     for (int i = 0; i < 8; ++i)
-        if (strides[i] < 0 || (strides[i] & (i < 6 ? in_mask : 7)) != 0) return HSTU_ERR_MISALIGNED;
+        if (strides[i] < 0 || (strides[i] & (i < 6 ? in_mask : out_mask)) != 0) return HSTU_ERR_MISALIGNED;
     return HSTU_OK;
 }
 
@@ -383,6 +392,38 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     // it an automatic choice falls back to the plain schedule, an explicit kv_splits > 1 is an error.
     Plan plan = make_plan(a);
     const bool ws_ok = a->workspace && (size_t)a->workspace_bytes >= plan.total();
+    if (a->dtype == HSTU_FP32) {
+        // the one use of the workspace that is not optional: rounded copies of the inputs
+        if (!ws_ok) return a->workspace ? HSTU_ERR_BAD_SHAPE : HSTU_ERR_NULL_POINTER;
+        char* cur = (char*)a->workspace + plan.total() - plan.cast_bytes;
+        const void* src[3] = {a->q, a->k, a->v};
+        const int64_t rs[3] = {a->q_row_stride, a->k_row_stride, a->v_row_stride};
+        const int64_t hs[3] = {a->q_head_stride, a->k_head_stride, a->v_head_stride};
+        const int64_t rows[3] = {a->total_q, a->total_kv, a->total_kv};
+        const int d[3] = {a->dqk, a->dqk, a->dv};
+        const char** dst[3] = {&p.q, &p.k, &p.v};
+        int64_t* prs[3] = {&p.q_rs, &p.k_rs, &p.v_rs};
+        int64_t* phs[3] = {&p.q_hs, &p.k_hs, &p.v_hs};
+        for (int i = 0; i < 3; ++i) {
+            cur = (char*)((reinterpret_cast<uintptr_t>(cur) + 255) & ~(uintptr_t)255);
+            const long long threads = (long long)rows[i] * a->heads * (d[i] / 8);
+            const long long blocks = (threads + 255) / 256;
+            if (blocks > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+            if (blocks > 0) {
+                hipLaunchKernelGGL(hstu::hstu_cast_f32_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const float*)src[i],
+                                   rs[i], hs[i], rows[i], a->heads, d[i], (_Float16*)cur);
+                hipError_t e = hipGetLastError();
+                if (e != hipSuccess) {
+                    set_last_error("cast kernel launch", e);
+                    return HSTU_ERR_LAUNCH;
+                }
+            }
+            *dst[i] = cur;
+            *prs[i] = (int64_t)a->heads * d[i];
+            *phs[i] = d[i];
+            cur += (size_t)rows[i] * a->heads * d[i] * 2;
+        }
+    }
     if (plan.splits > 1 && !ws_ok) {
         if (a->kv_splits > 1) return a->workspace ? HSTU_ERR_BAD_SHAPE : HSTU_ERR_NULL_POINTER;
         plan.splits = 1;
@@ -452,6 +493,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
         p.nitems = queue + 8 * 16;
     }
 
+    if (a->dtype == HSTU_FP32) return launch_mixed<hstu::Fp16F32>(p, a->dqk, a->dv, stream);
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
     if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
     return launch_dim<hstu::Fp8>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);

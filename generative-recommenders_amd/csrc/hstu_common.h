@@ -130,6 +130,10 @@ struct Fp16 {
         return r;
     }
 };
+// fp16 operands (rounded copies of fp32 inputs), fp32 output straight from the accumulators.
+struct Fp16F32 : Fp16 {
+    typedef float out_elem;
+};
 // OCP e4m3 (torch.float8_e4m3fn) inputs with per-tensor scales, bf16 output.  Both products run on
 // v_mfma_f32_32x32x16_fp8_fp8.  Q cannot be pre-scaled in 8 bits, so c1 (which here also carries
 // q_scale*k_scale) multiplies the accumulator.  P is kept in e4m3 as 16 * t * sigmoid: the factor 16 puts
@@ -656,10 +660,11 @@ template <class TT, int DT, int QT>
 __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int qt, char* o, int64_t orow0, int ql, int nq,
                                              int64_t o_rs, int64_t o_hs, int h, int g, float oscale,
                                              int dv_valid = 1 << 30) {
-    typedef typename TT::out_elem elem;  // 16 bits
+    typedef typename TT::out_elem elem;  // 16 bits, or float
     typedef __attribute__((ext_vector_type(4))) elem elem4;
+    constexpr int OES = sizeof(elem);
     if (ql >= nq) return;
-    char* op = o + ((orow0 + ql) * o_rs + (int64_t)h * o_hs) * 2 + g * 8;
+    char* op = o + ((orow0 + ql) * o_rs + (int64_t)h * o_hs) * OES + g * 4 * OES;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -668,8 +673,29 @@ __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int
             elem4 o4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) o4[i] = (elem)(oacc[dt][qt][r4 * 4 + i] * oscale);
-            *(elem4*)(op + (dt * 32 + r4 * 8) * 2) = o4;
+            *(elem4*)(op + (dt * 32 + r4 * 8) * OES) = o4;
         }
+}
+
+// dst[row][h][0..d) (dense, fp16) = src[row * rs + h * hs + 0..d) (fp32, strides in elements); 8 elements per thread.
+__global__ __launch_bounds__(256) void hstu_cast_f32_f16_kernel(const float* src, int64_t rs, int64_t hs, int64_t rows, int H,
+                                                                int d, _Float16* dst) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over rows * H * d / 8
+    const int d8 = d >> 3;
+    if (idx >= rows * H * d8) return;
+    const int c = (int)(idx % d8);
+    const int64_t rh = idx / d8;
+    const int h = (int)(rh % H);
+    const int64_t row = rh / H;
+    const float* sp = src + row * rs + (int64_t)h * hs + c * 8;
+    const f32x4_t a = *(const f32x4_t*)sp, b = *(const f32x4_t*)(sp + 4);
+    f16x8_t o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        o[i] = (_Float16)a[i];
+        o[4 + i] = (_Float16)b[i];
+    }
+    *(f16x8_t*)(dst + idx * 8) = o;
 }
 
 // The same store made row-contiguous: the wave first writes its 32 x DV output tile (16-bit elements) to its own

@@ -8,7 +8,7 @@ import torch
 
 from ..build import LIB_PATH
 
-HSTU_BF16, HSTU_FP16, HSTU_FP8_E4M3 = 0, 1, 2
+HSTU_BF16, HSTU_FP16, HSTU_FP8_E4M3, HSTU_FP32 = 0, 1, 2, 3
 
 
 class HstuFwdArgs(ctypes.Structure):
@@ -194,7 +194,9 @@ def _dtype_code(dt: torch.dtype) -> int:
         return HSTU_FP16
     if dt == torch.float8_e4m3fn:
         return HSTU_FP8_E4M3
-    raise RuntimeError(f"hstu_hip only supports fp16, bf16, and fp8_e4m3 data type, got {dt}")
+    if dt == torch.float32:
+        return HSTU_FP32
+    raise RuntimeError(f"hstu_hip only supports fp16, bf16, fp8_e4m3 and fp32 data type, got {dt}")
 
 
 def mha_fwd(

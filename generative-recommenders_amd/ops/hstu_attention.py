@@ -8,6 +8,8 @@ messages and output shapes.  Differences, all explicit:
   the reference, a scheduling hint (long sequences are started first) that never changes the result;
 * forward only -- inputs that require grad under ``torch.enable_grad()`` raise ``NotImplementedError``;
 * tensors must live on a HIP device; there is no CPU or PyTorch fallback;
+* fp32 q/k/v are rounded to fp16 inside the library (11-bit significand; the reference's Triton path multiplies in
+  tf32) and give an fp32 result;
 * fp8 (``torch.float8_e4m3fn``) q/k/v take per-tensor scales through ``q_scale``/``k_scale``/``v_scale``
   and give bf16 output, as the reference's native op does (``flash_common.cpp:596-607``);
 * ``tile_config`` / ``kv_splits`` choose the kernel and the split of the kv range over workgroups (0 = automatic);

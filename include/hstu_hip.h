@@ -23,8 +23,13 @@ extern "C" {
 #endif
 
 /* Element types of q/k/v.  Output is the same type, except FP8_E4M3 inputs give BF16 output
- * (flash_common.cpp:596-607). */
-enum HstuDtype { HSTU_BF16 = 0, HSTU_FP16 = 1, HSTU_FP8_E4M3 = 2 };
+ * (flash_common.cpp:596-607).
+ * FP32 (accepted by the reference's PyTorch and Triton backends, hstu_attention_test.py:270-274; not by its native
+ * op): the library first rounds q, k, v to fp16 copies in `workspace` (an 11-bit significand, one bit more than the
+ * tf32 products of the reference's Triton path; magnitudes beyond 65504 overflow), runs the fp16 kernel and stores
+ * the fp32 accumulators unrounded.  Needs the workspace, tile config 0 or 1, rows 16-byte aligned (strides multiples
+ * of 4 elements). */
+enum HstuDtype { HSTU_BF16 = 0, HSTU_FP16 = 1, HSTU_FP8_E4M3 = 2, HSTU_FP32 = 3 };
 
 /* Status codes.  0 is success; the library never throws or aborts. */
 enum HstuStatus {

@@ -338,6 +338,36 @@ def test_unequal_and_narrow_head_dims(pkg, dev, dqk, dv, dtype):
     assert_parity(got, O.cached_hstu_mha_per_sequence(200, alpha, dq.float(), k.float(), v.float(), offs, t), "delta")
 
 
+@pytest.mark.parametrize("dqk,dv", [(16, 16), (32, 64), (64, 64), (128, 128), (128, 32)])
+def test_fp32_inputs(pkg, dev, dqk, dv):
+    """fp32 q/k/v (the other dtype of the reference's test grid, hstu_attention_test.py:270-274): rounded to fp16
+    inside the library, fp32 out.  The error against the fp32 oracle is the fp16 rounding of the operands and of P,
+    two orders of magnitude inside the bf16 bar; strided column slices of one buffer are read in place."""
+    _announce("fp32", dqk, dv)
+    lengths = [300, 0, 64, 129, 17]
+    q, k, v, offs, t = make_case(3000 + dqk + dv, lengths, 2, dqk, dv, targets=[20, 0, 3, 0, 5], dtype=torch.float32)
+    N, alpha = 300, 1.0 / dqk**0.5
+    for w, c in [(0, 0), (50, 4)]:
+        got = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, w, c, 0, 0)
+        assert got.dtype == torch.float32 and got.shape == (sum(lengths), 2, dv)
+        ref = _ref_full(q, k, v, offs, t, N, alpha, w, c, 0)
+        assert_parity(got, ref, f"w={w} c={c}", rel_tol=2e-3)
+    fused = torch.cat([q, k, v], dim=2).to(dev)
+    got2 = pkg.hstu_mha(N, alpha, fused[:, :, :dqk], fused[:, :, dqk : 2 * dqk], fused[:, :, 2 * dqk :], offs.to(dev),
+                        num_targets=t.to(dev), max_attn_len=50, contextual_seq_len=4)
+    torch.cuda.synchronize()
+    assert torch.equal(got2, got)
+    delta = 16
+    lengths = np.array([200, 16, 77, 130])
+    q, k, v, offs, t = make_case(4000 + dqk + dv, lengths, 2, dqk, dv, targets=[delta] * 4, dtype=torch.float32)
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(4)])
+    dq = q[idx].contiguous()
+    got = pkg.delta_hstu_mha(200, alpha, dq.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev))
+    torch.cuda.synchronize()
+    assert got.dtype == torch.float32
+    assert_parity(got, O.cached_hstu_mha_per_sequence(200, alpha, dq, k, v, offs, t), "delta", rel_tol=2e-3)
+
+
 def test_invariants_on_device(pkg, dev):
     """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
     permuting two targets permutes the outputs (stu_test.py:180-321)."""
@@ -428,7 +458,9 @@ def test_wrapper_rejects_what_it_cannot_do(pkg, dev):
     with pytest.raises(AssertionError):
         pkg.hstu_mha(32, 0.1, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), causal=False)
     with pytest.raises(RuntimeError):
-        pkg.hstu_mha(32, 0.1, q.float().to(dev), k.float().to(dev), v.float().to(dev), offs.to(dev))
+        pkg.hstu_mha(32, 0.1, q.double().to(dev), k.double().to(dev), v.double().to(dev), offs.to(dev))
+    with pytest.raises(NotImplementedError):  # fp32 runs on the generic kernel only
+        pkg.hstu_mha(32, 0.1, q.float().to(dev), k.float().to(dev), v.float().to(dev), offs.to(dev), tile_config=2)
     qg = q.to(dev).requires_grad_()
     with pytest.raises(NotImplementedError):
         pkg.hstu_mha(32, 0.1, qg, k.to(dev), v.to(dev), offs.to(dev))

@@ -98,6 +98,9 @@ def test_check_args_status_codes(backend):
     assert chk(q=None) == -1
     assert chk(seq_offsets=None) == -1
     assert chk(dtype=7) == -2
+    assert chk(dtype=3) == 0  # fp32: rounded to fp16 inside the library
+    assert chk(dtype=3, tile_config=3) == -6
+    assert chk(dtype=3, q_row_stride=4 * 128 + 4) == 0 and chk(dtype=3, q_row_stride=4 * 128 + 2) == -4
     assert chk(dqk=48, dv=48) == -3
     assert chk(dqk=64, dv=128) == 0  # unequal dims run on tile config 1 ...
     assert chk(dqk=64, dv=128, tile_config=2) == -6  # ... only
