@@ -43,18 +43,36 @@ __global__ __launch_bounds__(256) void hstu_jagged_copy_kernel(const JaggedCopyP
     const int64_t r1 = r0 + ROWS < len_l + len_r ? r0 + ROWS : len_l + len_r;
     const int64_t vec_per_row = p.row_bytes / VEC;
     const int64_t total = (r1 - r0) * vec_per_row;
-    for (int64_t i = threadIdx.x; i < total; i += 256) {
-        const int64_t r = r0 + i / vec_per_row;
-        const int64_t c = (i % vec_per_row) * VEC;
-        char* part = r < len_l ? p.left + (ol + r) * p.left_rs : p.right + (orr + r - len_l) * p.right_rs;
-        char* whole = p.joined + (ol + orr + r) * p.joined_rs;
-        char* src = SPLIT ? whole : part;
-        char* dst = SPLIT ? part : whole;
-        if (VEC == 16) *(v16*)(dst + c) = *(const v16*)(src + c);
-        else if (VEC == 8) *(int64_t*)(dst + c) = *(const int64_t*)(src + c);
-        else if (VEC == 4) *(int*)(dst + c) = *(const int*)(src + c);
-        else if (VEC == 2) *(short*)(dst + c) = *(const short*)(src + c);
-        else dst[c] = src[c];
+    // four independent accesses per thread and round, loads first: a cold copy needs many bytes in flight
+    for (int64_t i0 = threadIdx.x; i0 < total; i0 += 1024) {
+        char* src[4];
+        char* dst[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t i = i0 + j * 256;
+            const int64_t ii = i < total ? i : i0;  // lanes past the end repeat their first access
+            const int64_t r = r0 + ii / vec_per_row;
+            const int64_t c = (ii % vec_per_row) * VEC;
+            char* part = r < len_l ? p.left + (ol + r) * p.left_rs : p.right + (orr + r - len_l) * p.right_rs;
+            char* whole = p.joined + (ol + orr + r) * p.joined_rs;
+            src[j] = (SPLIT ? whole : part) + c;
+            dst[j] = (SPLIT ? part : whole) + c;
+        }
+        if (VEC == 16) {
+            v16 x[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[j] = *(const v16*)src[j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *(v16*)dst[j] = x[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (VEC == 8) *(int64_t*)dst[j] = *(const int64_t*)src[j];
+                else if (VEC == 4) *(int*)dst[j] = *(const int*)src[j];
+                else if (VEC == 2) *(short*)dst[j] = *(const short*)src[j];
+                else *dst[j] = *src[j];
+            }
+        }
     }
 }
 
