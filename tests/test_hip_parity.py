@@ -368,6 +368,26 @@ def test_fp32_inputs(pkg, dev, dqk, dv):
     assert_parity(got, O.cached_hstu_mha_per_sequence(200, alpha, dq, k, v, offs, t), "delta", rel_tol=2e-3)
 
 
+def test_work_lists_beyond_the_class_cache(pkg, dev):
+    """More candidate row blocks per XCD (600 pairs x 64 blocks) than the plan kernel remembers between its two
+    walks: the tail of the candidates is classified twice.  Many tiny sequences, two long ones, one over-long one
+    (clamped to max_seq_len like everywhere else)."""
+    _announce("plan kernel beyond cache")
+    B, H, D, N = 1200, 4, 32, 8192
+    rng = np.random.default_rng(4321)
+    lengths = rng.integers(0, 40, size=B)
+    lengths[17], lengths[900], lengths[1199] = 3000, 8192, 700
+    q, k, v, offs, t = make_case(777, lengths, H, D, targets=np.minimum(lengths, rng.integers(0, 5, size=B)))
+    alpha = 1.0 / D**0.5
+    got = pkg.hstu_mha(N, alpha, q.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev), max_attn_len=1000,
+                       sort_by_length=True, tile_config=3)
+    torch.cuda.synchronize()
+    from generative_recommenders_amd.ops import hip_backend as hb
+
+    assert hb.plan_for(B, H, D, D, int(offs[-1]), int(offs[-1]), N, tile_config=3, sort_by_length=True) == (3, 1)
+    assert_parity(got, _ref_full(q, k, v, offs, t, N, alpha, 1000, 0, 0), "many sequences")
+
+
 def test_invariants_on_device(pkg, dev):
     """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
     permuting two targets permutes the outputs (stu_test.py:180-321)."""
