@@ -388,6 +388,29 @@ def test_work_lists_beyond_the_class_cache(pkg, dev):
     assert_parity(got, _ref_full(q, k, v, offs, t, N, alpha, 1000, 0, 0), "many sequences")
 
 
+@pytest.mark.parametrize("cfg", [2, 3])
+def test_delta_with_more_users_than_resident_workgroups(pkg, dev, cfg):
+    """Delta form with work lists and counters (several items per resident workgroup, ragged histories, window and
+    contextual prefix), which the small delta cases never reach."""
+    _announce("delta persistent", cfg)
+    B, H, D, delta = 600, 2, 32, 128 if cfg == 3 else 256
+    rng = np.random.default_rng(99)
+    lengths = rng.integers(0, 400, size=B) + delta + 3
+    lengths[5] = 2500
+    q, k, v, offs, t = make_case(555, lengths, H, D, targets=[delta] * B)
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(B)])
+    dq = q[idx].contiguous()
+    N, alpha = int(lengths.max()), 1.0 / D**0.5
+    from generative_recommenders_amd.ops import hip_backend as hb
+
+    assert hb.plan_for(B, H, D, D, B * delta, int(offs[-1]), N, delta_size=delta, tile_config=cfg) == (cfg, 1)
+    got = pkg.delta_hstu_mha(N, alpha, dq.to(dev), k.to(dev), v.to(dev), offs.to(dev), num_targets=t.to(dev), max_attn_len=300,
+                             contextual_seq_len=3, tile_config=cfg)
+    torch.cuda.synchronize()
+    ref = O.cached_hstu_mha_per_sequence(N, alpha, dq.float(), k.float(), v.float(), offs, t, 300, 3)
+    assert_parity(got, ref, "delta, many users")
+
+
 def test_invariants_on_device(pkg, dev):
     """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
     permuting two targets permutes the outputs (stu_test.py:180-321)."""
