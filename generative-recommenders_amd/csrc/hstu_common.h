@@ -149,6 +149,17 @@ struct Fp8 {
     static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
     }
+    // Four of these operands side by side are one operand of v_mfma_f32_32x32x64_f8f6f4, which runs at twice the
+    // rate of the 16-deep instruction (the only 8-bit rate that reaches the part's fp8 peak).  Which 32 of the 64
+    // k positions a lane group supplies does not matter as long as A and B agree, so the 8-byte pieces that the
+    // 16-deep scheme loads are simply used four at a time.
+    static __device__ __forceinline__ f32x16_t mfma64(const vec8 (&a)[4], const vec8 (&b)[4], f32x16_t c) {
+        typedef __attribute__((ext_vector_type(4))) long l4;
+        typedef __attribute__((ext_vector_type(8))) int i8;
+        const l4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(__builtin_bit_cast(i8, av), __builtin_bit_cast(i8, bv), c, 0, 0, 0, 0, 0,
+                                                               0);
+    }
     static __device__ __forceinline__ float silu(float raw, float c1) {
         const float t = raw * c1;
         const float e = __builtin_amdgcn_exp2f(t);

@@ -96,8 +96,11 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     // registers biased by VBIAS so that VOFF - VBIAS + slot and tile offsets fit the immediate as well.
     constexpr int VBIAS = (NSLOT * (KTILE + VTILE) > 65536) ? 32768 : 0;
     static_assert(VOFF >= VBIAS && VOFF - VBIAS + NSLOT * VTILE <= 65536 && NSLOT * KTILE <= 65536, "LDS immediates");
-    constexpr int NOPS = NS * KS + NS * 2 * DT;   // MFMAs of one matrix phase
-    constexpr int PD = NOPS >= 16 ? 6 : 4;        // operands in flight
+    // 8-bit operands: four 16-deep operands make one 64-deep MFMA at twice the rate (needs dqk % 64 == 0 and a
+    // 64-row kv tile)
+    constexpr bool WIDE = ES == 1 && DQK % 64 == 0 && BN == 64;
+    constexpr int NOPS = WIDE ? (NS * KS + NS * 2 * DT) / 4 : NS * KS + NS * 2 * DT;   // MFMAs of one matrix phase
+    constexpr int PD = NOPS >= 16 ? 6 : 4;        // operands in flight (16-deep scheme)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -241,26 +244,53 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         for (int sub = 0; sub < NS; ++sub) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[sub][r] = 0.f;
+            if constexpr (WIDE) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                vec8 a = *HSTU_LDS(const vec8, kt + sub * 32 * KROW + kaddr[ks]);
-                s[sub] = TT::mfma(a, qreg[ks], s[sub]);
+                for (int k4 = 0; k4 < KS / 4; ++k4) {
+                    vec8 a[4], b[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        a[j] = *HSTU_LDS(const vec8, kt + sub * 32 * KROW + kaddr[4 * k4 + j]);
+                        b[j] = qreg[4 * k4 + j];
+                    }
+                    s[sub] = TT::mfma64(a, b, s[sub]);
+                }
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    vec8 a = *HSTU_LDS(const vec8, kt + sub * 32 * KROW + kaddr[ks]);
+                    s[sub] = TT::mfma(a, qreg[ks], s[sub]);
+                }
             }
         }
     };
     // O^T += V^T P^T only (after the last step), V slot chosen at run time.
     auto gemm2_only = [&](int vslot) __attribute__((always_inline)) {
         const char* vt = smem + (VOFF - VBIAS) + vslot * VTILE;
+        if constexpr (WIDE) {
 #pragma unroll
-        for (int sub = 0; sub < NS; ++sub)
+            for (int dt = 0; dt < DT; ++dt) {
+                vec8 a[4], b[4];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const char* vb = vt + (sub * 32 + tt * 16) * VROW;
-                    vec8 a = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
-                    oacc[dt][0] = TT::mfma(a, pb[sub][tt], oacc[dt][0]);
+                for (int j = 0; j < 4; ++j) {  // j = 2 sub + tt: the whole 64-row tile in one MFMA
+                    const char* vb = vt + ((j >> 1) * 32 + (j & 1) * 16) * VROW;
+                    a[j] = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+                    b[j] = pb[j >> 1][j & 1];
                 }
+                oacc[dt][0] = TT::mfma64(a, b, oacc[dt][0]);
+            }
+        } else {
+#pragma unroll
+            for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        const char* vb = vt + (sub * 32 + tt * 16) * VROW;
+                        vec8 a = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+                        oacc[dt][0] = TT::mfma(a, pb[sub][tt], oacc[dt][0]);
+                    }
+        }
     };
     // Full matrix phase of list entry i (SLOT = i % 3): second product of entry i-1 interleaved with the
     // first product of entry i, plus this wave's share of the step's copies.
@@ -270,6 +300,49 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         constexpr int SLOT = decltype(slot_c)::value;
         const char* kt = smem + SLOT * KTILE;
         const char* vt = smem + (VOFF - VBIAS) + ((SLOT + NSLOT - 1) % NSLOT) * VTILE;
+        if constexpr (WIDE) {
+            // MFMA m: even m -> second product, dv tile m/2, all four (sub, tt) quarters of the kv tile at once;
+            //         odd m  -> first product, (k slab of 64, sub) = ((m/2)/NS, (m/2) % NS).
+            // The operands of MFMA m+1 are requested before MFMA m is issued.
+            auto load_group = [&](int m, vec8 (&a)[4]) __attribute__((always_inline)) {
+                const int o = m >> 1;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if ((m & 1) == 0) {
+                        const char* vb = vt + ((j >> 1) * 32 + (j & 1) * 16) * VROW;
+                        a[j] = read_vt_operand<TT>(vb + vaddr[0][o], vb + vaddr[1][o]);
+                    } else {
+                        a[j] = *HSTU_LDS(const vec8, kt + (o % NS) * 32 * KROW + kaddr[4 * (o / NS) + j]);
+                    }
+                }
+            };
+#pragma unroll
+            for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[sub][r] = 0.f;
+            vec8 fa[2][4];
+            load_group(0, fa[0]);
+#pragma unroll
+            for (int m = 0; m < NOPS; ++m) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (m + 1 < NOPS) load_group(m + 1, fa[(m + 1) & 1]);
+                const int o = m >> 1;
+                if ((m & 1) == 0) {
+                    vec8 b[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) b[j] = pb[j >> 1][j & 1];
+                    oacc[o][0] = TT::mfma64(fa[m & 1], b, oacc[o][0]);
+                } else {
+                    vec8 b[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) b[j] = qreg[4 * (o / NS) + j];
+                    s[o % NS] = TT::mfma64(fa[m & 1], b, s[o % NS]);
+                }
+                if (m % (NOPS / NPW) == (NOPS / NPW) - 1) issue_copy(slot_c, m / (NOPS / NPW));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            return;
+        }
         auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
             const int o = k >> 1;
             if ((k & 1) == 0) {
