@@ -24,7 +24,7 @@ PEAK_HBM_GBS = 8000.0
 HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced against HBM bandwidth
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"headline": 2.416e9, "cfg2": 0.827e9, "cfg3": 1.383e9, "cfg4": 0.249e9, "cfg5": 2.278e9,
+MEASURED_TRAFFIC_BYTES = {"headline": 2.414e9, "cfg2": 0.827e9, "cfg3": 1.383e9, "cfg4": 0.249e9, "cfg5": 2.281e9,
                           "kvcat": 0.173e9, "kvtail": 0.0168e9}
 
 
