@@ -411,6 +411,28 @@ def test_delta_with_more_users_than_resident_workgroups(pkg, dev, cfg):
     assert_parity(got, ref, "delta, many users")
 
 
+def test_long_sequences_32k(pkg, dev):
+    """max_seq_len = 32768, the length of the reference's long-sequence test (hstu_attention_test.py:296-323).  The
+    oracle checks the last 512 rows of every sequence (its cached-query form costs O(512 n) instead of O(n^2)); the
+    three kernels, written independently, must agree on all rows."""
+    _announce("32k")
+    N, H, D, delta = 32768, 1, 64, 512
+    lengths = np.array([32768, 20000, 700])
+    tg = np.array([32, 7, 0])
+    q, k, v, offs, t = make_case(3232, lengths, H, D, targets=tg)
+    alpha = 1.0 / D**0.5
+    outs = {cfg: _run_full(pkg, dev, q, k, v, offs, t, N, alpha, 0, 0, 0, cfg) for cfg in (1, 2, 3)}
+    idx = torch.cat([torch.arange(int(offs[b + 1]) - delta, int(offs[b + 1])) for b in range(3)])
+    ref = O.cached_hstu_mha_per_sequence(N, alpha, q[idx].float(), k.float(), v.float(), offs, t)
+    for cfg, out in outs.items():
+        assert_parity(out[idx.to(dev)], ref, f"tail rows, cfg {cfg}")
+    assert_parity(outs[2], outs[1].float(), "cfg 2 vs cfg 1", rel_tol=3e-3)
+    assert_parity(outs[3], outs[1].float(), "cfg 3 vs cfg 1", rel_tol=3e-3)
+    win = _run_full(pkg, dev, q, k, v, offs, t, N, alpha, 1000, 5, 0, 0)
+    ref_w = O.cached_hstu_mha_per_sequence(N, alpha, q[idx].float(), k.float(), v.float(), offs, t, 1000, 5)
+    assert_parity(win[idx.to(dev)], ref_w, "tail rows, window + contextual")
+
+
 def test_invariants_on_device(pkg, dev):
     """Size-independent properties: 1/N rescale is exact, batches and heads are independent,
     permuting two targets permutes the outputs (stu_test.py:180-321)."""
