@@ -166,12 +166,13 @@ struct Plan {
     int cfg;               // tile configuration, 1-based
     int splits;            // workgroups per row block along kv (1 = no split)
     int chunk;             // kv tiles per run when split
-    size_t queue_bytes;    // work-item counters and list lengths of the persistent kernels, at the start of the workspace
-    size_t items_bytes;    // work lists, behind the partial outputs (8 lists of {b * H + h, row block})
-    size_t order_bytes;    // sequence ranking, behind the counters
-    size_t counts_bytes;   // runs per row block, behind the ranking
-    size_t partial_bytes;  // fp32 partial outputs of the runs, 256-byte aligned behind the counts
-    size_t cast_bytes;     // fp16 copies of fp32 q, k, v, each 256-byte aligned, at the very end
+    // the workspace, in this order:
+    size_t queue_bytes;    // work-item counters and list lengths of the persistent kernels
+    size_t order_bytes;    // sequence ranking
+    size_t counts_bytes;   // runs per row block of a kv-split
+    size_t partial_bytes;  // fp32 partial outputs of the runs (256-byte aligned: 256 bytes of slack are added)
+    size_t items_bytes;    // work lists: 8 lists of {b * H + h, row block}
+    size_t cast_bytes;     // fp16 copies of fp32 q, k, v, each 256-byte aligned
     size_t total() const {
         return queue_bytes + order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0) + items_bytes + cast_bytes;
     }
@@ -460,7 +461,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     const int grid_per_xcd = (int)(slots < resident ? slots : resident);
     if (cfg < 2 || slots <= grid_per_xcd) queue = nullptr;  // every workgroup has exactly one item
     int* items = nullptr;
-    if (queue && plan.items_bytes > 0 && ws_bytes >= plan.total()) items = (int*)(ws + plan.total() - plan.items_bytes);
+    if (queue && plan.items_bytes > 0 && ws_bytes >= plan.total()) items = (int*)(ws + plan.total() - plan.cast_bytes - plan.items_bytes);
     // Equal-length sequences (every one as long as max_seq_len allows): dealing the items with a fixed stride is
     // perfectly balanced and keeps all workgroups of an XCD on the same (sequence, head) pair at the same time,
     // which measures 4-5 % faster than the counter; any other batch needs the counter for balance.
