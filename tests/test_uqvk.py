@@ -1,0 +1,183 @@
+"""hstu_compute_uqvk: the oracle against independent statements on the CPU, the HIP / hipBLASLt path against the
+oracle on the GPU.  Tolerance for bf16 / fp16 results (rounded once at the end, fp32 accumulation): relative
+Frobenius error <= 1e-2 and max-abs error <= 2e-2 * max|ref| against the fp32 oracle."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import uqvk_oracle as U
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _inputs(seed, L, d_model, H, attn, hidden, dtype):
+    g = torch.Generator().manual_seed(seed)
+    n_out = (2 * hidden + 2 * attn) * H
+    x = (torch.randn((L, d_model), generator=g) * 1.5 + 0.3).to(dtype)
+    nw = (1.0 + 0.1 * torch.randn(d_model, generator=g)).to(dtype)
+    nb = (0.1 * torch.randn(d_model, generator=g)).to(dtype)
+    w = (torch.randn((d_model, n_out), generator=g) / d_model**0.5).to(dtype)
+    b = (0.1 * torch.randn(n_out, generator=g)).to(dtype)
+    return x, nw, nb, w, b
+
+
+# ---------------------------------------------------------------- oracle, CPU
+
+
+def test_oracle_layer_norm_matches_the_formula_written_out():
+    x, nw, nb, _, _ = _inputs(1, 37, 96, 2, 8, 8, torch.float32)
+    got = U.layer_norm(x, nw, nb, 1e-6).double()
+    assert torch.allclose(got, U.layer_norm_by_hand(x, nw, nb, 1e-6), atol=1e-5)
+    # a layer norm does not see a positive rescaling or a shift of its input
+    assert torch.allclose(U.layer_norm(3.0 * x + 7.0, nw, nb, 1e-9).double(), got, atol=1e-4)
+
+
+def test_oracle_uqvk_against_pieces_written_by_hand():
+    L, d, H, attn, hidden = 21, 64, 3, 8, 16
+    x, nw, nb, w, b = _inputs(2, L, d, H, attn, hidden, torch.float32)
+    u, q, k, v = U.compute_uqvk(x, nw, nb, 1e-6, H, attn, hidden, w, b)
+    full = U.layer_norm_by_hand(x, nw, nb, 1e-6) @ w.double() + b.double()
+    hu, ha = hidden * H, attn * H
+    zu = full[:, :hu]
+    assert torch.allclose(u.double(), zu / (1 + torch.exp(-zu)), atol=1e-4)
+    assert torch.allclose(v.double(), full[:, hu : 2 * hu].reshape(L, H, hidden), atol=1e-4)
+    assert torch.allclose(q.double(), full[:, 2 * hu : 2 * hu + ha].reshape(L, H, attn), atol=1e-4)
+    assert torch.allclose(k.double(), full[:, 2 * hu + ha :].reshape(L, H, attn), atol=1e-4)
+    assert float(F.silu(torch.tensor(0.0))) == 0.0 and abs(float(F.silu(torch.tensor(30.0))) - 30.0) < 1e-6
+
+
+def test_uqvk_library_exports_and_struct_mirror():
+    import __graft_entry__
+
+    __graft_entry__.load_package()
+    from generative_recommenders_amd.ops import hstu_compute as hc
+
+    header = open(os.path.join(ROOT, "include", "hstu_uqvk.h")).read()
+    declared = set(re.findall(r"\b(hstu_uqvk_\w+)\s*\(", re.sub(r"/\*.*?\*/", "", header, flags=re.S)))
+    assert declared == set(hc.EXPORTS)
+    L = hc.lib()
+    for name in hc.EXPORTS:
+        assert hasattr(L, name)
+    body = header[header.index("typedef struct HstuUqvkArgs {") : header.index("} HstuUqvkArgs;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S).replace("typedef struct HstuUqvkArgs {", "")
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if decl:
+            parts = decl.split(",")
+            names.append(re.findall(r"(\w+)\s*$", parts[0].strip())[0])
+            names += [p.strip() for p in parts[1:]]
+    assert names == [f[0] for f in hc.HstuUqvkArgs._fields_]
+    # validation happens before anything touches the device
+    assert L.hstu_uqvk_forward(None, None) == -1
+    a = hc.HstuUqvkArgs()
+    a.rows, a.d_model, a.heads, a.attn_dim, a.hidden_dim = 4, 64, 2, 8, 8
+    assert L.hstu_uqvk_forward(ctypes.byref(a), None) == -1  # pointers missing
+    a.heads = 0
+    assert L.hstu_uqvk_forward(ctypes.byref(a), None) == -5
+    assert L.hstu_uqvk_layer_norm(None, 64, None, None, 1e-5, None, 64, 4, 60, 0, None) == -5  # d_model not a multiple of 8
+    assert L.hstu_uqvk_layer_norm(None, 64, None, None, 1e-5, None, 64, 0, 64, 0, None) == 0
+    src = open(os.path.join(ROOT, "generative-recommenders_amd", "ops", "hstu_compute.py")).read()
+    assert "oracle" not in src
+
+
+# ---------------------------------------------------------------- GPU
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    import __graft_entry__
+
+    __graft_entry__.load_package()
+    from generative_recommenders_amd.ops import hstu_compute
+
+    return hstu_compute
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return torch.device("cuda:0")
+
+
+def _close(got, ref, what):
+    got, ref = got.float().cpu(), ref.float()
+    assert got.shape == ref.shape, f"{what}: {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), what
+    rel = float((got - ref).norm() / ref.norm())
+    worst = float((got - ref).abs().max()) / float(ref.abs().max())
+    assert rel <= 1e-2 and worst <= 2e-2, f"{what}: relative {rel:.3e}, max-abs / max|ref| {worst:.3e}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,d_model", [(1, 64), (130, 512), (1000, 128), (77, 1024), (5, 4096), (64, 8)])
+def test_layer_norm_kernel(pkg, dev, L, d_model, dtype):
+    print(f"[case] layer norm {L} {d_model} {dtype}", flush=True)
+    x, nw, nb, _, _ = _inputs(L + d_model, L, d_model, 1, 8, 8, dtype)
+    got = pkg.layer_norm(x.to(dev), nw.to(dev), nb.to(dev), 1e-6)
+    torch.cuda.synchronize()
+    _close(got, U.layer_norm_by_hand(x, nw, nb, 1e-6), "layer norm")
+    wide = torch.cat([x, x], dim=1).to(dev)  # a column slice: row stride != width
+    got2 = pkg.layer_norm(wide[:, :d_model], nw.to(dev), nb.to(dev), 1e-6)
+    torch.cuda.synchronize()
+    assert torch.equal(got2, got)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,d_model,H,attn,hidden", [(300, 512, 4, 128, 128), (1, 64, 1, 16, 16), (1000, 128, 2, 32, 64), (257, 256, 4, 64, 32)])
+def test_compute_uqvk(pkg, dev, L, d_model, H, attn, hidden, dtype):
+    """Against the fp32 oracle, and tightly against the oracle with the reference's one intermediate rounding (the
+    normalised x in the input type)."""
+    print(f"[case] uqvk {L} {d_model} {H} {attn} {hidden} {dtype}", flush=True)
+    x, nw, nb, w, b = _inputs(L + d_model + attn, L, d_model, H, attn, hidden, dtype)
+    u, q, k, v = pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, attn, hidden, w.to(dev), b.to(dev))
+    torch.cuda.synchronize()
+    assert u.shape == (L, hidden * H) and q.shape == (L, H, attn) and k.shape == (L, H, attn) and v.shape == (L, H, hidden)
+    assert u.dtype == dtype and q.stride(2) == 1 and (L == 1 or q.stride(0) == (2 * hidden + 2 * attn) * H)
+    for name, got, ref in zip("uqkv", (u, q, k, v), U.compute_uqvk(x, nw, nb, 1e-6, H, attn, hidden, w, b)):
+        _close(got, ref, name)
+    for name, got, ref in zip("uqkv", (u, q, k, v), U.compute_uqvk(x, nw, nb, 1e-6, H, attn, hidden, w, b, round_normed_to=dtype)):
+        got, ref = got.float().cpu(), ref.float()
+        assert float((got - ref).norm() / ref.norm()) <= 4e-3, name
+
+
+@pytest.mark.gpu
+def test_uqvk_feeds_attention_in_place(pkg, dev):
+    """q, k, v are column slices of the projection's output; hstu_mha reads them where they are."""
+    import __graft_entry__
+    from oracle import hstu_oracle as O
+
+    top = __graft_entry__.load_package()
+    print("[case] uqvk -> hstu_mha", flush=True)
+    lengths = [200, 0, 64, 37]
+    offs = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int64)
+    L, d_model, H, D = int(offs[-1]), 256, 2, 64
+    x, nw, nb, w, b = _inputs(99, L, d_model, H, D, D, torch.bfloat16)
+    u, q, k, v = pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, D, D, w.to(dev), b.to(dev))
+    out = top.hstu_mha(200, 0.125, q, k, v, offs.to(dev))
+    torch.cuda.synchronize()
+    ref = O.hstu_mha_per_sequence(200, 0.125, q.float().cpu(), k.float().cpu(), v.float().cpu(), offs)
+    err = float((out.float().cpu() - ref).norm() / ref.norm())
+    assert err <= 1e-2, err
+
+
+@pytest.mark.gpu
+def test_uqvk_wrapper_rejections(pkg, dev):
+    x, nw, nb, w, b = [t.to(dev) for t in _inputs(5, 16, 64, 2, 8, 8, torch.bfloat16)]
+    with pytest.raises(AssertionError, match="uvqk_weight must be"):
+        pkg.hstu_compute_uqvk(x, nw, nb, 1e-6, 2, 8, 16, w, b)
+    with pytest.raises(RuntimeError):
+        pkg.hstu_compute_uqvk(x.float(), nw.float(), nb.float(), 1e-6, 2, 8, 8, w.float(), b.float())
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_compute_uqvk(x.clone().requires_grad_(), nw, nb, 1e-6, 2, 8, 8, w, b)
+    empty = pkg.hstu_compute_uqvk(x[:0], nw, nb, 1e-6, 2, 8, 8, w, b)
+    assert empty[0].shape == (0, 16) and empty[1].shape == (0, 2, 8)
