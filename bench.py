@@ -25,7 +25,8 @@ HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced ag
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
 MEASURED_TRAFFIC_BYTES = {"headline": 2.414e9, "cfg2": 0.827e9, "cfg3": 1.383e9, "cfg4": 0.249e9, "cfg5": 2.281e9,
-                          "kvcat": 0.173e9, "kvtail": 0.0168e9}
+                          "kvcat": 0.173e9, "kvtail": 0.0168e9, "uqvk": 5.549e9, "layernorm": 1.074e9, "output": 5.839e9,
+                          "normmul": 2.684e9}
 
 
 def run_gpu(wl, args, pkg, workloads, torch):
@@ -184,6 +185,88 @@ def run_jagged(name, args, pkg, torch):
     print(json.dumps(line))
 
 
+def run_linear(name, args, pkg, torch):
+    """The dense steps either side of the attention at the headline's token count (524288 rows, d_model 512, H=4,
+    attn = hidden = 128): `uqvk` = layer norm + projection + bias + SiLU(u) (hstu_compute_uqvk), `layernorm` = its
+    layer-norm kernel alone, `output` = norm * u, concatenation, projection + residual (hstu_compute_output with the
+    STU layer's flags), `normmul` = its norm-multiply-concatenate kernel alone."""
+    from generative_recommenders_amd.ops import hstu_compute
+
+    from oracle import output_oracle, uqvk_oracle
+
+    dev = torch.device("cuda:0")
+    L, d_model, H, D = 64 * 8192, 512, 4, 128
+    n_out = 4 * D * H
+    g = torch.Generator(device=dev).manual_seed(1000)
+
+    def rnd(*shape, scale=1.0, shift=0.0):
+        return (torch.randn(shape, device=dev, generator=g) * scale + shift).to(torch.bfloat16)
+
+    x = rnd(L, d_model, scale=1.5, shift=0.3)
+    if name in ("uqvk", "layernorm"):
+        nw, nb = rnd(d_model, scale=0.1, shift=1.0), rnd(d_model, scale=0.1)
+        w, b = rnd(d_model, n_out, scale=1.0 / d_model**0.5), rnd(n_out, scale=0.1)
+        if name == "uqvk":
+            step = lambda: hstu_compute.hstu_compute_uqvk(x, nw, nb, 1e-6, H, D, D, w, b)  # noqa: E731
+            cpu = lambda r: uqvk_oracle.compute_uqvk(x[:r].float().cpu(), nw.float().cpu(), nb.float().cpu(), 1e-6, H, D, D, w.float().cpu(), b.float().cpu())  # noqa: E731
+            flops, nbytes = 2.0 * L * d_model * n_out, 2.0 * (L * d_model + d_model * n_out + L * n_out)
+            kernel = "hstu_layer_norm_kernel + 2 hipBLASLt GEMMs (bias, bias + SiLU epilogues)"
+            metric = "hstu_compute_uqvk fwd TFLOP/s (524288 tokens, d_model 512 -> 2048)"
+        else:
+            step = lambda: hstu_compute.layer_norm(x, nw, nb, 1e-6)  # noqa: E731
+            cpu = lambda r: uqvk_oracle.layer_norm(x[:r].float().cpu(), nw.float().cpu(), nb.float().cpu(), 1e-6)  # noqa: E731
+            flops, nbytes = 0.0, 2.0 * 2 * L * d_model
+            kernel, metric = "hstu_layer_norm_kernel", "layer norm GB/s (524288 rows of 512 bf16)"
+    else:
+        attn, u = rnd(L, H * D, scale=0.1), rnd(L, H * D, scale=0.5)
+        nw, nb = rnd(H * D, scale=0.1, shift=1.0), rnd(H * D, scale=0.1)
+        w = rnd(3 * H * D, d_model, scale=1.0 / (3 * H * D) ** 0.5)
+        if name == "output":
+            step = lambda: hstu_compute.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, D, 0.0, False, True, True, "none", False, False)  # noqa: E731
+            cpu = lambda r: output_oracle.compute_output(attn[:r].float().cpu(), u[:r].float().cpu(), x[:r].float().cpu(), nw.float().cpu(), nb.float().cpu(), w.float().cpu(), 1e-6, concat_u=True, concat_x=True)  # noqa: E731
+            flops, nbytes = 2.0 * L * 3 * H * D * d_model, 2.0 * (2 * L * H * D + 2 * L * d_model + 3 * H * D * d_model)
+            kernel = "hstu_norm_mul_kernel + hipBLASLt GEMM (residual as C operand)"
+            metric = "hstu_compute_output fwd TFLOP/s (524288 tokens, 3 x 512 -> 512)"
+        else:
+            step = lambda: hstu_compute.norm_mul_dropout(attn, u, nw, nb, 1e-6, 0.0, False, False, True, True, "none")  # noqa: E731
+            cpu = lambda r: output_oracle.norm_mul(attn[:r].float().cpu(), u[:r].float().cpu(), nw.float().cpu(), nb.float().cpu(), 1e-6, concat_u=True, concat_x=True)  # noqa: E731
+            flops, nbytes = 0.0, 2.0 * (2 + 3) * L * H * D
+            kernel, metric = "hstu_norm_mul_kernel", "norm * u + concatenation GB/s (524288 rows, 2 x 512 in, 3 x 512 out, bf16)"
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    wall_ms, ev_ms = timed_steps(step, args, torch, flush=False)
+    tflops = flops / (ev_ms * 1e-3) / 1e12
+    gbs = nbytes / (ev_ms * 1e-3) / 1e9
+    if flops > 0:
+        roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                "frac": round(tflops / PEAK_TFLOPS["bf16"], 4)}
+        value, unit = round(tflops, 2), "TFLOP/s"
+    else:
+        roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
+        value, unit = round(gbs, 1), "GB/s"
+    roof.update({"traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel, "kernel_ms": round(ev_ms, 4),
+                 "algorithmic_flops": flops, "algorithmic_bytes": nbytes, "hbm_gbs_algorithmic": round(gbs, 1)})
+    line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic", "config": {"workload": name, "rows": L, "d_model": d_model, "heads": H, "attn_dim": D, "hidden_dim": D},
+            "roofline": roof}
+    if not args.no_cpu:
+        torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
+        rows = 32768
+        reps, t_used = 0, 0.0
+        while t_used < 10.0:
+            t0 = time.perf_counter()
+            cpu(rows)
+            t_used += time.perf_counter() - t0
+            reps += 1
+        frac = rows / L
+        cpu_val = (flops * frac * reps / t_used / 1e12) if flops > 0 else (nbytes * frac * reps / t_used / 1e9)
+        line["cpu_baseline"] = {"value": round(cpu_val, 4), "unit": unit, "cores": torch.get_num_threads(), "kind": "port",
+                                "sample": f"{reps} passes of the fp32 oracle over the first {rows} of {L} rows (conversion to fp32 included), {t_used:.1f} s"}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,7 +298,8 @@ def main():
     from generative_recommenders_amd import workloads
 
     jagged = args.workload in ("kvcat", "kvtail")
-    wl = None if jagged else workloads.make_workload(args.workload)
+    producer = args.workload in ("uqvk", "layernorm", "output", "normmul")
+    wl = None if jagged or producer else workloads.make_workload(args.workload)
     if wl is not None and wl.dtype == "fp32":
         print("bench.py: cfg1 is the CPU correctness case, not a GPU bench workload", file=sys.stderr)
         sys.exit(2)
@@ -228,6 +312,9 @@ def main():
         del src, dst
     if jagged:
         run_jagged(args.workload, args, pkg, torch)
+        return
+    if producer:
+        run_linear(args.workload, args, pkg, torch)
         return
     wall_ms, ev_ms = run_gpu(wl, args, pkg, workloads, torch)
     flops = workloads.algorithmic_flops(wl)

@@ -1,4 +1,4 @@
-"""Compile ``csrc/`` into ``csrc/libhstu_hip.so`` and ``csrc/libhstu_uqvk.so`` with hipcc for gfx950 (cross-compiles
+"""Compile ``csrc/`` into ``csrc/libhstu_hip.so`` and ``csrc/libhstu_linear.so`` with hipcc for gfx950 (cross-compiles
 without a GPU)."""
 
 import os
@@ -9,7 +9,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(_HERE), "include")
 LIB_PATH = os.path.join(CSRC, "libhstu_hip.so")
-UQVK_LIB_PATH = os.path.join(CSRC, "libhstu_uqvk.so")  # separate: it links hipBLASLt, the attention library does not
+LINEAR_LIB_PATH = os.path.join(CSRC, "libhstu_linear.so")  # separate: it links hipBLASLt, the attention library does not
 
 # -packed-fp32-ops off: hipcc must not fuse scalar float code into v_pk_*_f32 on this hardware pool.
 HIPCC_FLAGS = [
@@ -34,7 +34,7 @@ def build_library(verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)
     if verbose:
         print(" ".join(cmd))
-    cmd = [hipcc] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC, os.path.join(CSRC, "hstu_uqvk.hip"), "-o", UQVK_LIB_PATH, "-lhipblaslt"]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC, os.path.join(CSRC, "hstu_linear.hip"), "-o", LINEAR_LIB_PATH, "-lhipblaslt"]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)

@@ -1,0 +1,465 @@
+// C ABI of libhstu_linear.so: layer norm and norm-multiply-concatenate kernels + hipBLASLt GEMMs with fused bias /
+// SiLU epilogues and the residual as C operand.
+// Declarations and the reference interfaces they replace are in include/hstu_linear.h.
+#include "hstu_linear.h"
+
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <cstdio>
+#include <map>
+#include <mutex>
+#include <tuple>
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+
+thread_local char g_last_error[256] = "";
+
+// Sum over the 64 lanes of a wave, result in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+    return v;
+}
+
+// One wave per row, rows dealt to the waves of the grid with a stride.  A lane holds NCH chunks of 8 elements
+// (chunk c of the row goes to lane c % 64), loaded once; mean and variance in fp32 (two passes over the
+// registers, as torch's layer_norm does), weight and bias loaded once per wave.
+template <class V8, int NCH>
+__global__ __launch_bounds__(256) void hstu_layer_norm_kernel(const char* x, int64_t x_rs, const char* weight, const char* bias,
+                                                              float eps, char* out, int64_t out_rs, int64_t rows, int d) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    const int chunks = d >> 3;
+    float w[NCH][8], b[NCH][8];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = lane + 64 * i;
+        if (c < chunks) {
+            const V8 wv = *(const V8*)(weight + (int64_t)c * 16), bv = *(const V8*)(bias + (int64_t)c * 16);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                w[i][j] = (float)wv[j];
+                b[i][j] = (float)bv[j];
+            }
+        }
+    }
+    const float inv_d = 1.0f / (float)d;
+    for (int64_t r = wave; r < rows; r += nwaves) {
+        float v[NCH][8];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = lane + 64 * i;
+            if (c < chunks) {
+                const V8 xv = *(const V8*)(x + (r * x_rs + (int64_t)c * 8) * 2);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    v[i][j] = (float)xv[j];
+                    sum += v[i][j];
+                }
+            }
+        }
+        const float mean = wave_sum(sum) * inv_d;
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i)
+            if (lane + 64 * i < chunks)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sq += (v[i][j] - mean) * (v[i][j] - mean);
+        const float rstd = __builtin_amdgcn_rsqf(wave_sum(sq) * inv_d + eps);
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = lane + 64 * i;
+            if (c < chunks) {
+                V8 o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = (decltype(o[0] + o[0]))((v[i][j] - mean) * rstd * w[i][j] + b[i][j]);
+                *(V8*)(out + (r * out_rs + (int64_t)c * 8) * 2) = o;
+            }
+        }
+    }
+}
+
+int launch_layer_norm(const void* x, int64_t x_rs, const void* weight, const void* bias, float eps, void* out, int64_t out_rs,
+                      int64_t rows, int d, int dtype, hipStream_t stream) {
+    if (rows < 0 || d <= 0 || (d & 7) != 0 || d > 4096 || x_rs < d || out_rs < d || (x_rs & 7) != 0 || (out_rs & 7) != 0) return -5;
+    if (dtype != 0 && dtype != 1) return -2;
+    if (rows == 0) return 0;
+    if (!x || !weight || !bias || !out) return -1;
+    if ((((uintptr_t)x | (uintptr_t)weight | (uintptr_t)bias | (uintptr_t)out) & 15) != 0) return -4;
+    long long blocks = (rows + 3) / 4;
+    if (blocks > 256 * 16) blocks = 256 * 16;  // 16 four-wave workgroups per CU keep the loads in flight
+    const int nch = (d / 8 + 63) / 64;
+#define HSTU_LN(V8, N)                                                                                                          \
+    hipLaunchKernelGGL((hstu_layer_norm_kernel<V8, N>), dim3((unsigned)blocks), dim3(256), 0, stream, (const char*)x, x_rs,         \
+                       (const char*)weight, (const char*)bias, eps, (char*)out, out_rs, rows, d)
+    if (dtype == 0) {
+        if (nch <= 1) HSTU_LN(bf16x8_t, 1); else if (nch <= 2) HSTU_LN(bf16x8_t, 2); else if (nch <= 4) HSTU_LN(bf16x8_t, 4); else HSTU_LN(bf16x8_t, 8);
+    } else {
+        if (nch <= 1) HSTU_LN(f16x8_t, 1); else if (nch <= 2) HSTU_LN(f16x8_t, 2); else if (nch <= 4) HSTU_LN(f16x8_t, 4); else HSTU_LN(f16x8_t, 8);
+    }
+#undef HSTU_LN
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        snprintf(g_last_error, sizeof(g_last_error), "layer norm kernel launch: %s", hipGetErrorString(e));
+        return -7;
+    }
+    return 0;
+}
+
+// ---- norm * u, concatenated with the copied blocks ------------------------------------------------------------------
+struct NormMulParams {
+    const char *attn, *u, *weight, *bias;
+    char* joined;
+    int64_t attn_rs, u_rs, joined_rs, rows;  // strides in elements
+    float eps;
+    int d, group_lanes;                      // row width; lanes per head (group norm)
+    int off_u, off_x, off_y;                 // column offsets of the blocks in `joined`, -1 = block absent
+    int silu_u, mul_act;
+};
+
+__device__ __forceinline__ float sigmoid_f(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+
+// One wave per row as in the layer norm kernel.  GROUP: statistics per head (aligned groups of `group_lanes` lanes hold
+// one head's chunks, so the sums run over xor distances below group_lanes) and one weight / bias per head.
+template <class V8, int NCH, bool GROUP>
+__global__ __launch_bounds__(256) void hstu_norm_mul_kernel(NormMulParams p) {
+    typedef decltype(V8{}[0] + V8{}[0]) E;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * 4;
+    const int chunks = p.d >> 3;
+    float w[NCH][GROUP ? 1 : 8], b[NCH][GROUP ? 1 : 8];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = lane + 64 * i;
+        if (c < chunks) {
+            if constexpr (GROUP) {
+                const int head = c / p.group_lanes;
+                w[i][0] = (float)((const E*)p.weight)[head];
+                b[i][0] = (float)((const E*)p.bias)[head];
+            } else {
+                const V8 wv = *(const V8*)(p.weight + (int64_t)c * 16), bv = *(const V8*)(p.bias + (int64_t)c * 16);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    w[i][j] = (float)wv[j];
+                    b[i][j] = (float)bv[j];
+                }
+            }
+        }
+    }
+    const float inv_n = GROUP ? 1.0f / (float)(p.group_lanes * 8) : 1.0f / (float)p.d;
+    for (int64_t r = wave; r < p.rows; r += nwaves) {
+        float v[NCH][8];
+        V8 uraw[NCH], xraw[NCH];
+        float sum[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = lane + 64 * i;
+            sum[i] = 0.f;
+            if (c < chunks) {
+                xraw[i] = *(const V8*)(p.attn + (r * p.attn_rs + (int64_t)c * 8) * 2);
+                uraw[i] = *(const V8*)(p.u + (r * p.u_rs + (int64_t)c * 8) * 2);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    v[i][j] = (float)xraw[i][j];
+                    sum[i] += v[i][j];
+                }
+            }
+        }
+        float mean[NCH], rstd[NCH];
+        if constexpr (GROUP) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                for (int d = 1; d < p.group_lanes; d <<= 1) sum[i] += __shfl_xor(sum[i], d, 64);
+                mean[i] = sum[i] * inv_n;
+            }
+        } else {
+            float t = 0.f;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) t += sum[i];
+            t = wave_sum(t) * inv_n;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) mean[i] = t;
+        }
+        float sq[NCH];
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            sq[i] = 0.f;
+            if (lane + 64 * i < chunks)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sq[i] += (v[i][j] - mean[i]) * (v[i][j] - mean[i]);
+        }
+        if constexpr (GROUP) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                for (int d = 1; d < p.group_lanes; d <<= 1) sq[i] += __shfl_xor(sq[i], d, 64);
+                rstd[i] = __builtin_amdgcn_rsqf(sq[i] * inv_n + p.eps);
+            }
+        } else {
+            float t = 0.f;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) t += sq[i];
+            t = __builtin_amdgcn_rsqf(wave_sum(t) * inv_n + p.eps);
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) rstd[i] = t;
+        }
+        char* orow = p.joined + r * p.joined_rs * 2;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = lane + 64 * i;
+            if (c < chunks) {
+                V8 y, ucopy = uraw[i];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float uf = (float)uraw[i][j];
+                    const float us = uf * sigmoid_f(uf);
+                    float mul = uf;
+                    if constexpr (GROUP) {
+                        if (p.silu_u) mul = us;
+                    } else {
+                        if (p.mul_act == HSTU_MUL_U_SIGMOID) mul = sigmoid_f(uf);
+                        if (p.mul_act == HSTU_MUL_U_SILU) mul = us;
+                    }
+                    if (p.silu_u) ucopy[j] = (E)us;
+                    y[j] = (E)(mul * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]));
+                }
+                if (p.off_u >= 0) *(V8*)(orow + ((int64_t)p.off_u + c * 8) * 2) = ucopy;
+                if (p.off_x >= 0) *(V8*)(orow + ((int64_t)p.off_x + c * 8) * 2) = xraw[i];
+                *(V8*)(orow + ((int64_t)p.off_y + c * 8) * 2) = y;
+            }
+        }
+    }
+}
+
+int output_blocks(const HstuOutputArgs* a) {
+    if (a->group_norm) return (a->concat_u && a->concat_x) ? 3 : 1;
+    return 1 + (a->concat_u ? 1 : 0) + (a->concat_x ? 1 : 0);
+}
+
+int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hipStream_t stream) {
+    if (a->rows < 0 || a->heads <= 0 || a->linear_dim <= 0) return -5;
+    const int64_t d64 = (int64_t)a->heads * a->linear_dim;
+    if (d64 > 4096 || (d64 & 7) != 0) return -5;
+    const int d = (int)d64, blocks = output_blocks(a);
+    if (a->attn_row_stride < d || a->u_row_stride < d || joined_rs < (int64_t)blocks * d) return -5;
+    if (((a->attn_row_stride | a->u_row_stride | joined_rs) & 7) != 0) return -4;
+    if (a->dtype != 0 && a->dtype != 1) return -2;
+    if (a->mul_u_activation < 0 || a->mul_u_activation > 2) return -5;
+    int group_lanes = 0;
+    if (a->group_norm) {
+        group_lanes = a->linear_dim / 8;
+        if ((a->linear_dim & 7) != 0 || group_lanes > 64 || (group_lanes & (group_lanes - 1)) != 0) return -6;
+    }
+    if (a->rows == 0) return 0;
+    if (!a->attn || !a->u || !a->norm_weight || !a->norm_bias || !joined) return -1;
+    if ((((uintptr_t)a->attn | (uintptr_t)a->u | (uintptr_t)joined) & 15) != 0) return -4;
+    if (!a->group_norm && (((uintptr_t)a->norm_weight | (uintptr_t)a->norm_bias) & 15) != 0) return -4;
+    NormMulParams p;
+    p.attn = (const char*)a->attn, p.u = (const char*)a->u, p.weight = (const char*)a->norm_weight, p.bias = (const char*)a->norm_bias;
+    p.joined = (char*)joined;
+    p.attn_rs = a->attn_row_stride, p.u_rs = a->u_row_stride, p.joined_rs = joined_rs, p.rows = a->rows;
+    p.eps = a->norm_eps, p.d = d, p.group_lanes = group_lanes;
+    const bool cu = blocks == 3 || (!a->group_norm && a->concat_u), cx = blocks == 3 || (!a->group_norm && a->concat_x);
+    p.off_u = cu ? 0 : -1;
+    p.off_x = cx ? (cu ? d : 0) : -1;
+    p.off_y = (blocks - 1) * d;
+    p.silu_u = a->silu_u ? 1 : 0, p.mul_act = a->mul_u_activation;
+    long long wgs = (a->rows + 3) / 4;
+    if (wgs > 256 * 16) wgs = 256 * 16;
+    const int nch = (d / 8 + 63) / 64;
+#define HSTU_NM(V8, N, G) hipLaunchKernelGGL((hstu_norm_mul_kernel<V8, N, G>), dim3((unsigned)wgs), dim3(256), 0, stream, p)
+#define HSTU_NM_N(V8, G)                                                                                                \
+    do {                                                                                                                \
+        if (nch <= 1) HSTU_NM(V8, 1, G); else if (nch <= 2) HSTU_NM(V8, 2, G); else if (nch <= 4) HSTU_NM(V8, 4, G); else HSTU_NM(V8, 8, G); \
+    } while (0)
+    if (a->dtype == 0) {
+        if (a->group_norm) HSTU_NM_N(bf16x8_t, true); else HSTU_NM_N(bf16x8_t, false);
+    } else {
+        if (a->group_norm) HSTU_NM_N(f16x8_t, true); else HSTU_NM_N(f16x8_t, false);
+    }
+#undef HSTU_NM_N
+#undef HSTU_NM
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        snprintf(g_last_error, sizeof(g_last_error), "norm-mul kernel launch: %s", hipGetErrorString(e));
+        return -7;
+    }
+    return 0;
+}
+
+// ---- hipBLASLt: out[rows, n] = epilogue(act[rows, k] @ W[k, n] (+ bias) (+ residual)) ----------------------------------
+// Row-major out[rows, n] with row stride ldd is the column-major matrix D[n, rows]; D = A * B with A = W seen
+// column-major ([n, k], leading dimension ldw) and B = act seen column-major ([k, rows], leading dimension ldact).
+// The bias runs along D's rows, which is what the BIAS epilogues broadcast; the residual is the C operand (beta = 1).
+constexpr size_t kGemmScratch = 64u << 20;
+enum GemmEpilogue { kEpiNone = 0, kEpiBias = 1, kEpiBiasSilu = 2 };
+
+struct GemmPlan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr, d = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;
+};
+
+struct GemmShape {
+    long long rows, ldw, ldact, ldres, ldd;
+    int k, n, dtype, epi, device;
+    bool operator<(const GemmShape& o) const {
+        return std::tie(rows, ldw, ldact, ldres, ldd, k, n, dtype, epi, device) <
+               std::tie(o.rows, o.ldw, o.ldact, o.ldres, o.ldd, o.k, o.n, o.dtype, o.epi, o.device);
+    }
+};
+
+std::mutex g_mutex;
+hipblasLtHandle_t g_handle = nullptr;
+std::map<GemmShape, GemmPlan> g_plans;
+
+int blaslt_fail(const char* what, hipblasStatus_t st) {
+    snprintf(g_last_error, sizeof(g_last_error), "%s: hipBLASLt status %d", what, (int)st);
+    return HSTU_LINEAR_ERR_BLASLT;
+}
+
+// `residual` (row stride ldres) may be null: then ldres must be 0 and beta is 0.
+int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const void* bias, const void* residual, int64_t ldres,
+         void* out, int64_t ldd, int64_t rows, int k, int n, int dtype, int epi, void* scratch, hipStream_t stream) {
+    if (n == 0 || rows == 0) return 0;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    hipblasStatus_t st;
+    if (!g_handle && (st = hipblasLtCreate(&g_handle)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtCreate", st);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    const GemmShape key{(long long)rows, (long long)ldw, (long long)ldact, (long long)ldres, (long long)ldd, k, n, dtype, epi, dev};
+    auto it = g_plans.find(key);
+    if (it == g_plans.end()) {
+        GemmPlan pl;
+        const hipDataType t = dtype == 0 ? HIP_R_16BF : HIP_R_16F;
+        if ((st = hipblasLtMatmulDescCreate(&pl.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F)) != HIPBLAS_STATUS_SUCCESS)
+            return blaslt_fail("hipblasLtMatmulDescCreate", st);
+        if (epi != kEpiNone) {
+            const hipblasLtEpilogue_t e = epi == kEpiBiasSilu ? HIPBLASLT_EPILOGUE_SWISH_BIAS_EXT : HIPBLASLT_EPILOGUE_BIAS;
+            st = hipblasLtMatmulDescSetAttribute(pl.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &e, sizeof(e));
+            if (st == HIPBLAS_STATUS_SUCCESS) {
+                const int32_t bt = (int32_t)t;
+                st = hipblasLtMatmulDescSetAttribute(pl.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt));
+            }
+            // the bias pointer takes part in the heuristic query; it is set again for every call below
+            if (st == HIPBLAS_STATUS_SUCCESS)
+                st = hipblasLtMatmulDescSetAttribute(pl.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+            if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmulDescSetAttribute", st);
+        }
+        if ((st = hipblasLtMatrixLayoutCreate(&pl.a, t, n, k, ldw)) != HIPBLAS_STATUS_SUCCESS ||
+            (st = hipblasLtMatrixLayoutCreate(&pl.b, t, k, rows, ldact)) != HIPBLAS_STATUS_SUCCESS ||
+            (st = hipblasLtMatrixLayoutCreate(&pl.c, t, n, rows, residual ? ldres : ldd)) != HIPBLAS_STATUS_SUCCESS ||
+            (st = hipblasLtMatrixLayoutCreate(&pl.d, t, n, rows, ldd)) != HIPBLAS_STATUS_SUCCESS)
+            return blaslt_fail("hipblasLtMatrixLayoutCreate", st);
+        hipblasLtMatmulPreference_t pref;
+        if ((st = hipblasLtMatmulPreferenceCreate(&pref)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("preference", st);
+        const uint64_t max_ws = kGemmScratch;
+        hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+        hipblasLtMatmulHeuristicResult_t res[1];
+        int found = 0;
+        st = hipblasLtMatmulAlgoGetHeuristic(g_handle, pl.desc, pl.a, pl.b, pl.c, pl.d, pref, 1, res, &found);
+        hipblasLtMatmulPreferenceDestroy(pref);
+        if (st != HIPBLAS_STATUS_SUCCESS || found < 1) return blaslt_fail("hipblasLtMatmulAlgoGetHeuristic", st);
+        pl.algo = res[0].algo;
+        pl.workspace = res[0].workspaceSize;
+        it = g_plans.emplace(key, pl).first;
+    }
+    GemmPlan& pl = it->second;
+    if (epi != kEpiNone) {
+        st = hipblasLtMatmulDescSetAttribute(pl.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+        if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("bias pointer", st);
+    }
+    const float one = 1.0f, beta = residual ? 1.0f : 0.0f;
+    st = hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out, pl.d, &pl.algo,
+                         scratch, pl.workspace, stream);
+    if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmul", st);
+    return 0;
+}
+
+size_t normed_bytes(const HstuUqvkArgs* a) { return (((size_t)a->rows * a->d_model * 2) + 255) & ~(size_t)255; }
+size_t joined_bytes(const HstuOutputArgs* a) {
+    return (((size_t)a->rows * output_blocks(a) * a->heads * a->linear_dim * 2) + 255) & ~(size_t)255;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* hstu_linear_last_error(void) { return g_last_error; }
+
+size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* a) {
+    if (!a || a->rows <= 0 || a->d_model <= 0) return 0;
+    return normed_bytes(a) + kGemmScratch;
+}
+
+int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight, const void* bias, float eps, void* out,
+                         int64_t out_row_stride, int64_t rows, int32_t d_model, int32_t dtype, void* stream) {
+    g_last_error[0] = 0;
+    return launch_layer_norm(x, x_row_stride, weight, bias, eps, out, out_row_stride, rows, d_model, dtype, (hipStream_t)stream);
+}
+
+int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
+    g_last_error[0] = 0;
+    if (!a) return -1;
+    if (a->rows < 0 || a->heads <= 0 || a->attn_dim <= 0 || a->hidden_dim <= 0 || a->d_model <= 0) return -5;
+    if (a->rows == 0) return 0;
+    if (!a->uvqk_weight || !a->uvqk_bias || !a->uvqk || !a->workspace) return -1;
+    if ((size_t)a->workspace_bytes < hstu_uqvk_workspace_bytes(a) || ((uintptr_t)a->workspace & 255) != 0) return -4;
+    if (a->rows > 0x7fffffffLL) return -5;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int n_u = a->hidden_dim * a->heads;
+    const int n_out = (2 * a->hidden_dim + 2 * a->attn_dim) * a->heads;
+    if ((n_u & 7) != 0 || (n_out & 7) != 0) return -4;  // column blocks start on 16-byte boundaries
+    void* normed = a->workspace;
+    void* scratch = (char*)a->workspace + normed_bytes(a);
+    int rc = launch_layer_norm(a->x, a->x_row_stride, a->norm_weight, a->norm_bias, a->norm_eps, normed, a->d_model, a->rows,
+                               a->d_model, a->dtype, stream);
+    if (rc != 0) return rc;
+    // u columns with SiLU in the epilogue, then v | q | k with the bias only
+    const char* w = (const char*)a->uvqk_weight;
+    const char* b = (const char*)a->uvqk_bias;
+    char* o = (char*)a->uvqk;
+    rc = gemm(normed, a->d_model, w, n_out, b, nullptr, 0, o, n_out, a->rows, a->d_model, n_u, a->dtype, kEpiBiasSilu, scratch, stream);
+    if (rc != 0) return rc;
+    return gemm(normed, a->d_model, w + (int64_t)n_u * 2, n_out, b + (int64_t)n_u * 2, nullptr, 0, o + (int64_t)n_u * 2, n_out, a->rows,
+                a->d_model, n_out - n_u, a->dtype, kEpiBias, scratch, stream);
+}
+
+size_t hstu_output_workspace_bytes(const HstuOutputArgs* a) {
+    if (!a || a->rows <= 0 || a->heads <= 0 || a->linear_dim <= 0) return 0;
+    return joined_bytes(a) + kGemmScratch;
+}
+
+int hstu_output_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_row_stride, void* stream) {
+    g_last_error[0] = 0;
+    if (!a) return -1;
+    return launch_norm_mul(a, joined, joined_row_stride, (hipStream_t)stream);
+}
+
+int hstu_output_forward(const HstuOutputArgs* a, void* stream_) {
+    g_last_error[0] = 0;
+    if (!a) return -1;
+    if (a->rows < 0 || a->heads <= 0 || a->linear_dim <= 0 || a->d_out <= 0 || (a->d_out & 7) != 0) return -5;
+    if (a->rows > 0x7fffffffLL || a->x_row_stride < a->d_out || (a->x_row_stride & 7) != 0) return -5;
+    if (a->rows == 0) return 0;
+    if (!a->x || !a->output_weight || !a->out || !a->workspace) return -1;
+    if ((((uintptr_t)a->x | (uintptr_t)a->output_weight | (uintptr_t)a->out) & 15) != 0) return -4;
+    if ((size_t)a->workspace_bytes < hstu_output_workspace_bytes(a) || ((uintptr_t)a->workspace & 255) != 0) return -4;
+    hipStream_t stream = (hipStream_t)stream_;
+    const int k = output_blocks(a) * a->heads * a->linear_dim;
+    void* joined = a->workspace;
+    void* scratch = (char*)a->workspace + joined_bytes(a);
+    int rc = launch_norm_mul(a, joined, k, stream);
+    if (rc != 0) return rc;
+    return gemm(joined, k, a->output_weight, a->d_out, nullptr, a->x, a->x_row_stride, a->out, a->d_out, a->rows, k, a->d_out, a->dtype,
+                kEpiNone, scratch, stream);
+}
+
+}  // extern "C"

@@ -1,9 +1,15 @@
-"""``hstu_compute_uqvk`` with the reference's signature: layer norm + uvqk projection + split + SiLU(u).
+"""``hstu_compute_uqvk``, ``hstu_compute_output`` and ``hstu_preprocess_and_attention`` with the reference's
+signatures (``generative_recommenders/ops/hstu_compute.py:54-104``, ``:107-214``, ``:217-334``).
 
-Mirrors ``generative_recommenders/ops/hstu_compute.py:54-104`` of the reference.  The layer norm is a hand-written
-gfx950 kernel; the projection is a plain GEMM and runs on hipBLASLt with the bias and, for the u columns, the SiLU
-in its epilogue (``csrc/hstu_uqvk.hip``, ``include/hstu_uqvk.h``).  ``u, q, k, v`` come back as column slices of one
-``[L, (2*hidden + 2*attn) * H]`` buffer, which ``hstu_mha`` / ``delta_hstu_mha`` read in place.
+``hstu_compute_uqvk``: layer norm + uvqk projection + split + SiLU(u).  The layer norm is a hand-written gfx950
+kernel; the projection is a plain GEMM and runs on hipBLASLt with the bias and, for the u columns, the SiLU in its
+epilogue.  ``u, q, k, v`` come back as column slices of one ``[L, (2*hidden + 2*attn) * H]`` buffer, which
+``hstu_mha`` / ``delta_hstu_mha`` read in place.
+
+``hstu_compute_output``: ``x + [u | attn | act(u) * norm(attn)] @ output_weight``.  One hand-written kernel
+normalises, multiplies and writes the concatenated operand; the product, with the residual as the GEMM's C operand,
+runs on hipBLASLt.  (``csrc/hstu_linear.hip``, ``include/hstu_linear.h``.)
+
 Forward only, device tensors only, bf16 or fp16; ``kernel`` is accepted and ignored.
 """
 
@@ -13,12 +19,12 @@ from typing import Optional, Tuple
 
 import torch
 
-from ..build import UQVK_LIB_PATH
+from ..build import LINEAR_LIB_PATH
 from ..common import HammerKernel
 
 
 class HstuUqvkArgs(ctypes.Structure):
-    """Mirror of ``HstuUqvkArgs`` in include/hstu_uqvk.h (field order and types must match)."""
+    """Mirror of ``HstuUqvkArgs`` in include/hstu_linear.h (field order and types must match)."""
 
     _fields_ = [
         ("x", ctypes.c_void_p),
@@ -40,18 +46,52 @@ class HstuUqvkArgs(ctypes.Structure):
     ]
 
 
-EXPORTS = ("hstu_uqvk_workspace_bytes", "hstu_uqvk_forward", "hstu_uqvk_layer_norm", "hstu_uqvk_last_error")
+class HstuOutputArgs(ctypes.Structure):
+    """Mirror of ``HstuOutputArgs`` in include/hstu_linear.h (field order and types must match)."""
+
+    _fields_ = [
+        ("attn", ctypes.c_void_p),
+        ("attn_row_stride", ctypes.c_int64),
+        ("u", ctypes.c_void_p),
+        ("u_row_stride", ctypes.c_int64),
+        ("x", ctypes.c_void_p),
+        ("x_row_stride", ctypes.c_int64),
+        ("norm_weight", ctypes.c_void_p),
+        ("norm_bias", ctypes.c_void_p),
+        ("norm_eps", ctypes.c_float),
+        ("output_weight", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("rows", ctypes.c_int64),
+        ("d_out", ctypes.c_int32),
+        ("heads", ctypes.c_int32),
+        ("linear_dim", ctypes.c_int32),
+        ("concat_u", ctypes.c_int32),
+        ("concat_x", ctypes.c_int32),
+        ("group_norm", ctypes.c_int32),
+        ("silu_u", ctypes.c_int32),
+        ("mul_u_activation", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_int64),
+    ]
+
+
+EXPORTS = (
+    "hstu_uqvk_workspace_bytes", "hstu_uqvk_forward", "hstu_uqvk_layer_norm", "hstu_output_workspace_bytes", "hstu_output_forward",
+    "hstu_output_norm_mul", "hstu_linear_last_error",
+)
+MUL_U_ACTIVATIONS = {"none": 0, "sigmoid": 1, "silu": 2}
 
 _lib: Optional[ctypes.CDLL] = None
 
 
 def lib() -> ctypes.CDLL:
-    """Load libhstu_uqvk.so.  Raises if it has not been built: there is no fallback path."""
+    """Load libhstu_linear.so.  Raises if it has not been built: there is no fallback path."""
     global _lib
     if _lib is None:
-        if not os.path.exists(UQVK_LIB_PATH):
-            raise RuntimeError(f"{UQVK_LIB_PATH} is missing: build it with __graft_entry__.build().  There is no fallback.")
-        L = ctypes.CDLL(UQVK_LIB_PATH)
+        if not os.path.exists(LINEAR_LIB_PATH):
+            raise RuntimeError(f"{LINEAR_LIB_PATH} is missing: build it with __graft_entry__.build().  There is no fallback.")
+        L = ctypes.CDLL(LINEAR_LIB_PATH)
         L.hstu_uqvk_workspace_bytes.restype = ctypes.c_size_t
         L.hstu_uqvk_workspace_bytes.argtypes = [ctypes.POINTER(HstuUqvkArgs)]
         L.hstu_uqvk_forward.restype = ctypes.c_int
@@ -61,7 +101,13 @@ def lib() -> ctypes.CDLL:
             ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_int64,
             ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p,
         ]
-        L.hstu_uqvk_last_error.restype = ctypes.c_char_p
+        L.hstu_output_workspace_bytes.restype = ctypes.c_size_t
+        L.hstu_output_workspace_bytes.argtypes = [ctypes.POINTER(HstuOutputArgs)]
+        L.hstu_output_forward.restype = ctypes.c_int
+        L.hstu_output_forward.argtypes = [ctypes.POINTER(HstuOutputArgs), ctypes.c_void_p]
+        L.hstu_output_norm_mul.restype = ctypes.c_int
+        L.hstu_output_norm_mul.argtypes = [ctypes.POINTER(HstuOutputArgs), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        L.hstu_linear_last_error.restype = ctypes.c_char_p
         _lib = L
     return _lib
 
@@ -71,8 +117,8 @@ _STATUS = {-1: ValueError, -2: RuntimeError, -4: RuntimeError, -5: ValueError, -
 
 def _raise_for_status(rc: int) -> None:
     if rc != 0:
-        extra = lib().hstu_uqvk_last_error().decode()
-        raise _STATUS.get(rc, RuntimeError)(f"hstu_uqvk: status {rc}" + (f" ({extra})" if extra else ""))
+        extra = lib().hstu_linear_last_error().decode()
+        raise _STATUS.get(rc, RuntimeError)(f"hstu_linear: status {rc}" + (f" ({extra})" if extra else ""))
 
 
 def _dtype_code(dt: torch.dtype) -> int:
@@ -80,7 +126,7 @@ def _dtype_code(dt: torch.dtype) -> int:
         return 0
     if dt == torch.float16:
         return 1
-    raise RuntimeError(f"hstu_uqvk only supports bf16 and fp16, got {dt}")
+    raise RuntimeError(f"hstu_compute only supports bf16 and fp16, got {dt}")
 
 
 def _check(x: torch.Tensor, *others: torch.Tensor) -> None:
@@ -157,3 +203,146 @@ def hstu_compute_uqvk(
         uvqk, [hidden_dim * num_heads, hidden_dim * num_heads, attn_dim * num_heads, attn_dim * num_heads], dim=1
     )
     return u, q.view(-1, num_heads, attn_dim), k.view(-1, num_heads, attn_dim), v.view(-1, num_heads, hidden_dim)
+
+
+def _rows_ok(t: torch.Tensor) -> torch.Tensor:
+    t = t.detach()
+    if t.stride(1) != 1 or (t.shape[0] > 1 and t.stride(0) % 8 != 0) or t.data_ptr() % 16 != 0:
+        t = t.contiguous()
+    return t
+
+
+def _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_dim, concat_u, concat_x, mul_u_activation_type,
+                 group_norm, silu_u) -> Tuple[HstuOutputArgs, tuple, int]:
+    torch._assert(attn.dim() == 2 and u.shape == attn.shape, "attn and u must be 2-D and of one shape")
+    torch._assert(attn.shape[1] == num_heads * linear_dim, "attn.shape[1] must equal num_heads * linear_dim")
+    torch._assert(mul_u_activation_type in MUL_U_ACTIVATIONS, "mul_u_activation_type must be none, sigmoid or silu")
+    norm_len = num_heads if group_norm else attn.shape[1]
+    torch._assert(norm_weight.shape == (norm_len,) and norm_bias.shape == (norm_len,), "norm_weight / norm_bias have the wrong length")
+    attn, u = _rows_ok(attn), _rows_ok(u)
+    nw, nb = norm_weight.detach().contiguous(), norm_bias.detach().contiguous()
+    a = HstuOutputArgs()
+    a.attn, a.attn_row_stride = attn.data_ptr(), max(attn.stride(0), attn.shape[1])
+    a.u, a.u_row_stride = u.data_ptr(), max(u.stride(0), u.shape[1])
+    a.norm_weight, a.norm_bias, a.norm_eps = nw.data_ptr(), nb.data_ptr(), norm_eps
+    a.rows, a.heads, a.linear_dim = attn.shape[0], num_heads, linear_dim
+    a.concat_u, a.concat_x, a.group_norm, a.silu_u = int(concat_u), int(concat_x), int(group_norm), int(silu_u)
+    a.mul_u_activation = MUL_U_ACTIVATIONS[mul_u_activation_type]
+    a.dtype = _dtype_code(attn.dtype)
+    if group_norm:
+        blocks = 3 if (concat_u and concat_x) else 1
+    else:
+        blocks = 1 + int(concat_u) + int(concat_x)
+    return a, (attn, u, nw, nb), blocks
+
+
+def _no_dropout(dropout_ratio: float, training: bool) -> None:
+    if training and dropout_ratio > 0.0:
+        raise NotImplementedError("the HIP backend implements the dropout-free forward only (training=False or dropout_ratio=0)")
+
+
+def norm_mul_dropout(
+    x: torch.Tensor, u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, dropout_ratio: float, training: bool,
+    silu_u: bool = False, concat_u: bool = False, concat_x: bool = False, mul_u_activation_type: str = "none",
+    group_norm: bool = False, num_heads: int = 1, linear_dim: int = -1,
+) -> torch.Tensor:
+    """``act(u) * norm(x)`` joined with the copied blocks (``ops/pytorch/pt_hstu_linear.py:24-85`` of the reference),
+    without dropout."""
+    _no_dropout(dropout_ratio, training)
+    _check(x, u, weight, bias)
+    if not group_norm:
+        num_heads, linear_dim = 1, x.shape[1]
+    a, keep, blocks = _output_args(x, u, weight, bias, eps, num_heads, linear_dim, concat_u, concat_x, mul_u_activation_type, group_norm, silu_u)
+    joined = torch.empty((x.shape[0], blocks * x.shape[1]), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
+        rc = lib().hstu_output_norm_mul(ctypes.byref(a), joined.data_ptr(), joined.shape[1], ctypes.c_void_p(stream))
+    _raise_for_status(rc)
+    return joined
+
+
+def hstu_compute_output(
+    attn: torch.Tensor,
+    u: torch.Tensor,
+    x: torch.Tensor,
+    norm_weight: torch.Tensor,
+    norm_bias: torch.Tensor,
+    norm_eps: float,
+    output_weight: torch.Tensor,
+    num_heads: int,
+    linear_dim: int,
+    dropout_ratio: float,
+    training: bool,
+    concat_u: bool,
+    concat_x: bool,
+    mul_u_activation_type: str,
+    group_norm: bool,
+    recompute_y_in_backward: bool,
+    kernel: HammerKernel = HammerKernel.HIP,
+) -> torch.Tensor:
+    """Returns ``x + joined @ output_weight`` of shape ``[L, d_model]``; ``recompute_y_in_backward`` concerns the
+    backward pass only and is ignored."""
+    _no_dropout(dropout_ratio, training)
+    torch._assert(x.dim() == 2 and x.shape[0] == attn.shape[0], "x must be 2-D with attn's row count")
+    _check(x, attn, u, norm_weight, norm_bias, output_weight)
+    a, keep, blocks = _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_dim, concat_u, concat_x,
+                                   mul_u_activation_type, group_norm, False)
+    torch._assert(output_weight.shape == (blocks * attn.shape[1], x.shape[1]), "output_weight must be [blocks * heads * linear_dim, d_model]")
+    xr, w = _rows_ok(x), output_weight.detach().contiguous()
+    out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    a.x, a.x_row_stride = xr.data_ptr(), max(xr.stride(0), xr.shape[1])
+    a.output_weight, a.out, a.d_out = w.data_ptr(), out.data_ptr(), x.shape[1]
+    if x.shape[0] > 0:
+        need = lib().hstu_output_workspace_bytes(ctypes.byref(a))
+        workspace = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
+        a.workspace, a.workspace_bytes = (workspace.data_ptr() + 255) & ~255, need
+        with torch.cuda.device(x.device):
+            stream = torch.cuda.current_stream(x.device).cuda_stream
+            rc = lib().hstu_output_forward(ctypes.byref(a), ctypes.c_void_p(stream))
+        _raise_for_status(rc)
+    return out
+
+
+def hstu_preprocess_and_attention(
+    x: torch.Tensor,
+    norm_weight: torch.Tensor,
+    norm_bias: torch.Tensor,
+    norm_eps: float,
+    num_heads: int,
+    attn_dim: int,
+    hidden_dim: int,
+    uvqk_weight: torch.Tensor,
+    uvqk_bias: torch.Tensor,
+    max_seq_len: int,
+    seq_offsets: torch.Tensor,
+    attn_alpha: float,
+    causal: bool,
+    num_targets: Optional[torch.Tensor],
+    max_attn_len: int,
+    contextual_seq_len: int,
+    recompute_uvqk_in_backward: bool,
+    recompute_normed_x_in_backward: bool,
+    sort_by_length: bool,
+    prefill: bool = False,
+    kernel: HammerKernel = HammerKernel.HIP,
+    enable_tma: Optional[bool] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """``hstu_compute_uqvk`` followed by ``hstu_mha`` on the views it returns; returns ``(u, attn_output, k, v)`` with
+    ``attn_output [L, hidden * H]``.  The ``recompute_*`` flags concern the backward pass only and are ignored."""
+    from .hstu_attention import hstu_mha
+
+    torch._assert(max_seq_len > 0, "max_seq_len must be larger than 0")
+    torch._assert(x.dim() == 2, "x must be 2-D")
+    torch._assert(x.shape[1] == uvqk_weight.shape[0], "x.shape[1] must equal uvqk_weight.shape[0]")
+    torch._assert(
+        uvqk_weight.shape[1] == 2 * num_heads * (hidden_dim + attn_dim),
+        "uvqk_weight.shape[1] must equal 2 * num_heads * (hidden_dim + attn_dim)",
+    )
+    torch._assert(causal is True, "only causal attention is supported.")
+    u, q, k, v = hstu_compute_uqvk(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, kernel)
+    attn_output = hstu_mha(
+        max_seq_len=max_seq_len, alpha=attn_alpha, q=q, k=k, v=v, seq_offsets=seq_offsets, causal=causal, dropout_pr=0.0,
+        training=False, num_targets=num_targets, max_attn_len=max_attn_len, contextual_seq_len=contextual_seq_len,
+        sort_by_length=sort_by_length, kernel=kernel,
+    ).view(-1, hidden_dim * num_heads)
+    return u, attn_output, k, v

@@ -1,0 +1,112 @@
+/*
+ * hstu_linear.h -- C ABI of libhstu_linear.so: the producer of q, k, v for the HSTU attention path on gfx950 and the
+ * consumer of its output.
+ *
+ * Producer: replaces `hstu_compute_uqvk` (generative_recommenders/ops/hstu_compute.py:54-104):
+ *     normed = layer_norm(x, weight, bias, eps)                 (fp32 statistics, result in x's type,
+ *                                                                ops/pytorch/pt_layer_norm.py:24-39)
+ *     uvqk   = uvqk_bias + normed @ uvqk_weight                 [L, (2*hidden + 2*attn) * H]
+ *     u, v, q, k = split(uvqk, [hidden*H, hidden*H, attn*H, attn*H]);  u = silu(u)
+ * All four results stay column slices of ONE [L, n_out] buffer -- the layout the attention entry points read in
+ * place through their row / head strides -- so nothing is copied on the way to `hstu_hip_mha_fwd`.
+ *
+ * The layer norm is a hand-written kernel (one wave per row, HBM-bound).  The matrix product is a plain GEMM and
+ * goes to hipBLASLt, with the bias and, for the u columns, the SiLU in the GEMM's epilogue.  This library is
+ * separate from libhstu_hip.so so that the attention library does not depend on hipBLASLt.
+ * Plain pointers and sizes; device pointers on the current HIP device; asynchronous on the stream given.
+ */
+#ifndef HSTU_LINEAR_H_
+#define HSTU_LINEAR_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Status codes: 0 ok; negative values as in hstu_hip.h (-1 NULL pointer, -2 dtype, -4 alignment, -5 shape,
+ * -6 unsupported, -7 HIP launch failure), -9 hipBLASLt failure (see hstu_linear_last_error()). */
+enum { HSTU_LINEAR_ERR_BLASLT = -9 };
+
+typedef struct HstuUqvkArgs {
+    const void* x;             /* [rows, d_model], bf16 or fp16, innermost stride 1 */
+    int64_t x_row_stride;      /* elements */
+    const void* norm_weight;   /* [d_model], same type */
+    const void* norm_bias;     /* [d_model] */
+    float norm_eps;
+    const void* uvqk_weight;   /* [d_model, n_out] row-major, dense */
+    const void* uvqk_bias;     /* [n_out] */
+    void* uvqk;                /* [rows, n_out] dense output: u | v | q | k column blocks, u already through SiLU */
+    int64_t rows;
+    int32_t d_model;           /* multiple of 8, at most 4096 */
+    int32_t heads, attn_dim, hidden_dim;  /* n_out = (2 * hidden_dim + 2 * attn_dim) * heads */
+    int32_t dtype;             /* 0 = bf16, 1 = fp16 (HstuDtype of hstu_hip.h) */
+    void* workspace;           /* hstu_uqvk_workspace_bytes() bytes, 256-byte aligned: the normalised x and the
+                                  GEMM's scratch */
+    int64_t workspace_bytes;
+} HstuUqvkArgs;
+
+size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* args);
+
+/* layer norm + GEMM + bias + split + SiLU(u), as described at the top. */
+int hstu_uqvk_forward(const HstuUqvkArgs* args, void* stream);
+
+/* Only the layer norm: out[r] = (x[r] - mean) * rsqrt(var + eps) * weight + bias, statistics in fp32
+ * (ops/pytorch/pt_layer_norm.py:24-39).  Strides in elements. */
+int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight, const void* bias, float eps, void* out,
+                         int64_t out_row_stride, int64_t rows, int32_t d_model, int32_t dtype, void* stream);
+
+/*
+ * Consumer: replaces `hstu_compute_output` (generative_recommenders/ops/hstu_compute.py:107-214) in its forward,
+ * dropout-free form, i.e. `pytorch_hstu_compute_output` (ops/pytorch/pt_hstu_linear.py:88-124):
+ *     y   = norm_mul(attn, u)                      (pt_hstu_linear.py:24-85, statistics and product in fp32)
+ *              layer norm : y = act(u) * layer_norm(attn) over the whole row, act in {none, sigmoid, silu};
+ *                           joined = [u] | [attn] | y, a block present when concat_u / concat_x is set
+ *              group norm : y = u * group_norm(attn) per head of linear_dim columns, one weight and bias per head;
+ *                           joined = u | attn | y only when concat_u AND concat_x, else y alone (as the reference)
+ *              silu_u     : layer norm: the copied u block goes through SiLU; group norm: u does before both uses
+ *     out = x + joined @ output_weight             [rows, d_out]
+ * The norm / multiply / concatenate step is one hand-written kernel (one wave per row, HBM-bound) that writes
+ * `joined` in the inputs' type; the product with the residual as the GEMM's C operand runs on hipBLASLt.
+ */
+enum { HSTU_MUL_U_NONE = 0, HSTU_MUL_U_SIGMOID = 1, HSTU_MUL_U_SILU = 2 };
+
+typedef struct HstuOutputArgs {
+    const void* attn;          /* [rows, heads * linear_dim], bf16 or fp16, innermost stride 1 */
+    int64_t attn_row_stride;   /* elements */
+    const void* u;             /* [rows, heads * linear_dim] */
+    int64_t u_row_stride;
+    const void* x;             /* [rows, d_out]: the residual */
+    int64_t x_row_stride;
+    const void* norm_weight;   /* layer norm: [heads * linear_dim]; group norm: [heads] */
+    const void* norm_bias;
+    float norm_eps;
+    const void* output_weight; /* [blocks * heads * linear_dim, d_out] row-major, dense; blocks = 1 + copied blocks */
+    void* out;                 /* [rows, d_out] dense */
+    int64_t rows;
+    int32_t d_out;             /* multiple of 8 */
+    int32_t heads, linear_dim; /* heads * linear_dim: multiple of 8, at most 4096; group norm: linear_dim / 8 a power of two <= 64 */
+    int32_t concat_u, concat_x, group_norm, silu_u;  /* 0 / 1 */
+    int32_t mul_u_activation;  /* HSTU_MUL_U_*; layer norm only */
+    int32_t dtype;             /* 0 = bf16, 1 = fp16 */
+    void* workspace;           /* hstu_output_workspace_bytes() bytes, 256-byte aligned: `joined` and the GEMM's scratch */
+    int64_t workspace_bytes;
+} HstuOutputArgs;
+
+size_t hstu_output_workspace_bytes(const HstuOutputArgs* args);
+
+/* norm_mul + concatenation + GEMM + residual, as described above. */
+int hstu_output_forward(const HstuOutputArgs* args, void* stream);
+
+/* Only the first step (`pytorch_norm_mul_dropout` without dropout, pt_hstu_linear.py:24-85): writes `joined`
+ * [rows, blocks * heads * linear_dim] with row stride `joined_row_stride` elements.  Reads attn, u, norm_weight,
+ * norm_bias, norm_eps, rows, heads, linear_dim, the five flags and dtype of `args`; the other fields are ignored. */
+int hstu_output_norm_mul(const HstuOutputArgs* args, void* joined, int64_t joined_row_stride, void* stream);
+
+const char* hstu_linear_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_LINEAR_H_ */

@@ -1,0 +1,236 @@
+"""hstu_compute_output: the oracle against independent statements on the CPU, the HIP / hipBLASLt path against the
+oracle on the GPU.  Inputs are uniform in [-0.1, 0.1] as in the reference's own test
+(ops/tests/hstu_compute_test.py:119-170).  Tolerance for bf16 / fp16 results (rounded once at the end, fp32
+accumulation): relative Frobenius error <= 1e-2 and max-abs error <= 2e-2 * max|ref| against the fp32 oracle; the
+concatenated operand's copied blocks are bit-exact."""
+
+import itertools
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import output_oracle as O
+from oracle import uqvk_oracle as U
+
+
+def _inputs(seed, N, H, linear_dim, D, blocks, group_norm, dtype):
+    g = torch.Generator().manual_seed(seed)
+    L = H * linear_dim
+
+    def uni(*shape):
+        return (torch.rand(shape, generator=g) * 0.2 - 0.1).to(dtype)
+
+    attn, u, x = uni(N, L), uni(N, L), uni(N, D)
+    nw, nb = uni(H if group_norm else L), uni(H if group_norm else L)
+    w = uni(blocks * L, D)
+    return attn, u, x, nw, nb, w
+
+
+def _blocks(concat_u, concat_x, group_norm):
+    if group_norm:
+        return 3 if (concat_u and concat_x) else 1
+    return 1 + int(concat_u) + int(concat_x)
+
+
+# ---------------------------------------------------------------- oracle, CPU
+
+
+def test_oracle_group_norm_matches_the_formula_written_out():
+    attn, u, _, nw, nb, _ = _inputs(1, 19, 3, 16, 8, 1, True, torch.float32)
+    got = O.norm_mul(attn, u, nw, nb, 1e-6, group_norm=True, num_heads=3, linear_dim=16).double()
+    assert torch.allclose(got, u.double() * O.group_norm_by_hand(attn, 3, 16, nw, nb, 1e-6), atol=1e-5)
+    # one head: a group norm with a scalar weight is the layer norm with that scalar in every column
+    got1 = O.norm_mul(attn, u, nw[:1], nb[:1], 1e-6, group_norm=True, num_heads=1, linear_dim=48).double()
+    ln = U.layer_norm_by_hand(attn, nw[:1].expand(48), nb[:1].expand(48), 1e-6)
+    assert torch.allclose(got1, u.double() * ln, atol=1e-5)
+
+
+@pytest.mark.parametrize("act", ["none", "sigmoid", "silu"])
+def test_oracle_layer_norm_mode_and_blocks(act):
+    attn, u, _, nw, nb, _ = _inputs(2, 11, 2, 16, 8, 1, False, torch.float32)
+    ud = u.double()
+    mul = {"none": ud, "sigmoid": 1 / (1 + torch.exp(-ud)), "silu": ud / (1 + torch.exp(-ud))}[act]
+    y = mul * U.layer_norm_by_hand(attn, nw, nb, 1e-6)
+    for cu, cx, silu_u in itertools.product((False, True), (False, True), (False, True)):
+        got = O.norm_mul(attn, u, nw, nb, 1e-6, silu_u=silu_u, concat_u=cu, concat_x=cx, mul_u_activation_type=act).double()
+        want = ([ud / (1 + torch.exp(-ud)) if silu_u else ud] if cu else []) + ([attn.double()] if cx else []) + [y]
+        assert got.shape[1] == 32 * len(want)
+        assert torch.allclose(got, torch.cat(want, dim=1), atol=1e-5), (cu, cx, silu_u)
+
+
+def test_oracle_group_norm_concatenates_only_with_both_flags():
+    attn, u, _, nw, nb, _ = _inputs(3, 7, 2, 8, 8, 1, True, torch.float32)
+    y = O.norm_mul(attn, u, nw, nb, 1e-6, group_norm=True, num_heads=2, linear_dim=8)
+    for cu, cx in ((True, False), (False, True)):
+        assert torch.equal(O.norm_mul(attn, u, nw, nb, 1e-6, concat_u=cu, concat_x=cx, group_norm=True, num_heads=2, linear_dim=8), y)
+    both = O.norm_mul(attn, u, nw, nb, 1e-6, concat_u=True, concat_x=True, group_norm=True, num_heads=2, linear_dim=8)
+    assert torch.equal(both, torch.cat([u, attn, y], dim=1))
+    silu = O.norm_mul(attn, u, nw, nb, 1e-6, silu_u=True, concat_u=True, concat_x=True, group_norm=True, num_heads=2, linear_dim=8)
+    assert torch.allclose(silu[:, :16], F.silu(u)) and torch.allclose(silu[:, 32:], F.silu(u) * (y / u), atol=1e-5)
+
+
+def test_oracle_output_with_a_selecting_weight():
+    """A one-hot output_weight picks single columns of the concatenated operand, so each block's place shows."""
+    N, H, ld, D = 9, 2, 8, 8
+    attn, u, x, nw, nb, _ = _inputs(4, N, H, ld, D, 3, False, torch.float32)
+    L = H * ld
+    w = torch.zeros((3 * L, D))
+    picks = [0, L - 1, L, 2 * L - 1, 2 * L, 3 * L - 1, 5, L + 5]
+    for col, row in enumerate(picks):
+        w[row, col] = 1.0
+    out = O.compute_output(attn, u, x, nw, nb, w, 1e-6, concat_u=True, concat_x=True)
+    y = (u.double() * U.layer_norm_by_hand(attn, nw, nb, 1e-6)).float()
+    joined = torch.cat([u, attn, y], dim=1)
+    assert torch.allclose(out, x + joined[:, picks], atol=1e-5)
+
+
+# ---------------------------------------------------------------- GPU
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    import __graft_entry__
+
+    __graft_entry__.load_package()
+    from generative_recommenders_amd.ops import hstu_compute
+
+    return hstu_compute
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return torch.device("cuda:0")
+
+
+def _close(got, ref, what):
+    got, ref = got.float().cpu(), ref.float()
+    assert got.shape == ref.shape, f"{what}: {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), what
+    rel = float((got - ref).norm() / ref.norm())
+    worst = float((got - ref).abs().max()) / float(ref.abs().max())
+    assert rel <= 1e-2 and worst <= 2e-2, f"{what}: relative {rel:.3e}, max-abs / max|ref| {worst:.3e}"
+
+
+NORM_MUL_CASES = [
+    # N, H, linear_dim, group_norm
+    (1000, 4, 128, False), (1000, 4, 128, True), (1, 1, 8, False), (3, 2, 8, True), (65, 3, 64, True), (130, 5, 24, False),
+    (37, 2, 512, True), (9, 8, 512, False), (21, 4, 256, False), (300, 16, 16, True),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,H,ld,group_norm", NORM_MUL_CASES)
+def test_norm_mul_kernel(pkg, dev, N, H, ld, group_norm, dtype):
+    L = H * ld
+    attn, u, _, nw, nb, _ = _inputs(N + L, N, H, ld, 8, 1, group_norm, dtype)
+    for cu, cx, silu_u, act in [(True, True, False, "none"), (False, False, False, "silu"), (True, False, True, "sigmoid"), (False, True, False, "none")]:
+        print(f"[case] norm_mul {N} {H} {ld} group={group_norm} {dtype} {cu} {cx} {silu_u} {act}", flush=True)
+        got = pkg.norm_mul_dropout(attn.to(dev), u.to(dev), nw.to(dev), nb.to(dev), 1e-6, 0.0, False, silu_u, cu, cx, act, group_norm, H, ld)
+        torch.cuda.synchronize()
+        ref = O.norm_mul(attn, u, nw, nb, 1e-6, silu_u, cu, cx, act, group_norm, H, ld)
+        _close(got, ref, "joined")
+        blocks = _blocks(cu, cx, group_norm)
+        assert got.shape == (N, blocks * L)
+        got = got.cpu()
+        if blocks == 3 or (not group_norm and cx):  # the attn block is a copy
+            off = L if (blocks == 3 or cu) else 0
+            assert torch.equal(got[:, off : off + L], attn)
+        if (blocks == 3 or (not group_norm and cu)) and not silu_u:
+            assert torch.equal(got[:, :L], u)
+
+
+OUTPUT_CASES = [
+    # N, H, linear_dim, D, concat_u, concat_x, act, group_norm      (first rows: the reference test's shapes)
+    (1000, 4, 128, 128, True, True, "none", False),
+    (1000, 4, 128, 128, False, True, "silu", False),
+    (1000, 4, 128, 128, True, False, "sigmoid", False),
+    (1000, 4, 128, 128, False, False, "none", False),
+    (1000, 4, 128, 128, True, True, "none", True),
+    (1000, 4, 128, 128, True, False, "none", True),
+    (4099, 4, 128, 512, True, True, "none", False),
+    (1, 2, 8, 8, True, True, "none", False),
+    (77, 2, 64, 72, False, True, "none", True),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,H,ld,D,cu,cx,act,group_norm", OUTPUT_CASES)
+def test_compute_output(pkg, dev, N, H, ld, D, cu, cx, act, group_norm, dtype):
+    print(f"[case] output {N} {H} {ld} {D} {cu} {cx} {act} group={group_norm} {dtype}", flush=True)
+    blocks = _blocks(cu, cx, group_norm)
+    attn, u, x, nw, nb, w = _inputs(N + D, N, H, ld, D, blocks, group_norm, dtype)
+    got = pkg.hstu_compute_output(attn.to(dev), u.to(dev), x.to(dev), nw.to(dev), nb.to(dev), 1e-6, w.to(dev), H, ld, 0.0, False,
+                                  cu, cx, act, group_norm, False)
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == (N, D)
+    kw = dict(concat_u=cu, concat_x=cx, mul_u_activation_type=act, group_norm=group_norm, num_heads=H, linear_dim=ld)
+    _close(got, O.compute_output(attn, u, x, nw, nb, w, 1e-6, **kw), "out vs fp32 oracle")
+    _close(got, O.compute_output(attn, u, x, nw, nb, w, 1e-6, round_joined_to=dtype, **kw), "out vs oracle with the operand rounded")
+    # the residual alone: a zero weight returns x bit for bit
+    zero = pkg.hstu_compute_output(attn.to(dev), u.to(dev), x.to(dev), nw.to(dev), nb.to(dev), 1e-6, torch.zeros_like(w).to(dev), H, ld,
+                                   0.3, False, cu, cx, act, group_norm, True)
+    assert torch.equal(zero.cpu(), x)
+
+
+@pytest.mark.gpu
+def test_output_takes_strided_views_and_rejects_what_it_cannot_do(pkg, dev):
+    N, H, ld, D = 50, 2, 64, 64
+    attn, u, x, nw, nb, w = [t.to(dev) for t in _inputs(5, N, H, ld, D, 3, False, torch.bfloat16)]
+    want = pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "none", False, False)
+    wide = torch.cat([u, attn, u], dim=1)  # u and attn as column slices of a wider buffer
+    got = pkg.hstu_compute_output(wide[:, H * ld : 2 * H * ld], wide[:, : H * ld], torch.cat([x, x], dim=1)[:, :D], nw, nb, 1e-6, w, H,
+                                  ld, 0.0, False, True, True, "none", False, False)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, ld, 0.3, True, True, True, "none", False, False)
+    with pytest.raises(AssertionError):
+        pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w[:-8], H, ld, 0.0, False, True, True, "none", False, False)
+    with pytest.raises(AssertionError):
+        pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "tanh", False, False)
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_compute_output(attn.clone().requires_grad_(), u, x, nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "none", False, False)
+    with pytest.raises(NotImplementedError):  # group norm over 3 chunks per head
+        pkg.norm_mul_dropout(attn[:, :48], u[:, :48], nw[:2], nb[:2], 1e-6, 0.0, False, group_norm=True, num_heads=2, linear_dim=24)
+    empty = pkg.hstu_compute_output(attn[:0], u[:0], x[:0], nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "none", False, False)
+    assert empty.shape == (0, D)
+
+
+@pytest.mark.gpu
+def test_preprocess_and_attention_then_output(pkg, dev):
+    """One STU layer's forward strung together (modules/stu.py:286-356 of the reference) against the oracles."""
+    import numpy as np
+
+    from oracle import hstu_oracle
+
+    H, Dh, d_model, B, N = 2, 64, 128, 5, 200
+    rng = np.random.default_rng(11)
+    lengths = rng.integers(20, N + 1, size=B)
+    offsets = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int64)
+    L = int(offsets[-1])
+    g = torch.Generator().manual_seed(12)
+    dt = torch.bfloat16
+    x = torch.randn((L, d_model), generator=g).to(dt)
+    nw, nb = (1 + 0.1 * torch.randn(d_model, generator=g)).to(dt), (0.1 * torch.randn(d_model, generator=g)).to(dt)
+    wq = (torch.randn((d_model, 4 * Dh * H), generator=g) / d_model**0.5).to(dt)
+    bq = (0.1 * torch.randn(4 * Dh * H, generator=g)).to(dt)
+    ow, ob = (1 + 0.1 * torch.randn(Dh * H, generator=g)).to(dt), (0.1 * torch.randn(Dh * H, generator=g)).to(dt)
+    wo = (torch.randn((3 * Dh * H, d_model), generator=g) / (3 * Dh * H) ** 0.5).to(dt)
+    alpha = 1.0 / Dh**0.5
+    print("[case] preprocess_and_attention + output", flush=True)
+    u, attn, k, v = pkg.hstu_preprocess_and_attention(
+        x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, Dh, Dh, wq.to(dev), bq.to(dev), N, offsets.to(dev), alpha, True, None, 0, 0,
+        False, False, False,
+    )
+    out = pkg.hstu_compute_output(attn, u, x.to(dev), ow.to(dev), ob.to(dev), 1e-6, wo.to(dev), H, Dh, 0.0, False, True, True, "none", False, False)
+    torch.cuda.synchronize()
+    assert attn.shape == (L, H * Dh) and k.shape == (L, H, Dh) and v.shape == (L, H, Dh)
+    ru, rq, rk, rv = U.compute_uqvk(x, nw, nb, 1e-6, H, Dh, Dh, wq, bq)
+    rattn = hstu_oracle.pytorch_hstu_mha(N, alpha, rq, rk, rv, offsets).reshape(L, H * Dh)
+    _close(attn, rattn, "attention output")
+    _close(out, O.compute_output(rattn, ru, x, ow, ob, wo, 1e-6, concat_u=True, concat_x=True, num_heads=H, linear_dim=Dh), "layer output")
