@@ -25,19 +25,30 @@ HIPCC_FLAGS = [
 ]
 
 
+def _run(cmd, verbose):
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + proc.stdout + proc.stderr)
+    if verbose:
+        print(" ".join(cmd))
+
+
 def build_library(verbose: bool = False) -> str:
-    """Always recompiles; returns the path of the shared library."""
+    """Always recompiles; returns the path of the attention library.  The translation units compile side by side
+    (forward, backward, dense steps), then libhstu_hip.so is linked from the first two."""
+    from concurrent.futures import ThreadPoolExecutor
+
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [hipcc] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC, os.path.join(CSRC, "hstu_api.hip"), "-o", LIB_PATH]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)
-    if verbose:
-        print(" ".join(cmd))
-    cmd = [hipcc] + HIPCC_FLAGS + ["-I", INCLUDE, "-I", CSRC, os.path.join(CSRC, "hstu_linear.hip"), "-o", LINEAR_LIB_PATH, "-lhipblaslt"]
-    proc = subprocess.run(cmd, capture_output=True, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + proc.stdout + proc.stderr)
-    if verbose:
-        print(" ".join(cmd))
+    common = [hipcc] + [f for f in HIPCC_FLAGS if f != "-shared"] + ["-I", INCLUDE, "-I", CSRC]
+    objs = [os.path.join(CSRC, "hstu_api.o"), os.path.join(CSRC, "hstu_bwd_api.o")]
+    jobs = [
+        common + ["-c", os.path.join(CSRC, "hstu_api.hip"), "-o", objs[0]],
+        common + ["-c", os.path.join(CSRC, "hstu_bwd_api.hip"), "-o", objs[1]],
+        common + ["-shared", os.path.join(CSRC, "hstu_linear.hip"), "-o", LINEAR_LIB_PATH, "-lhipblaslt"],
+    ]
+    with ThreadPoolExecutor(max_workers=3) as pool:
+        list(pool.map(lambda c: _run(c, verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC"] + objs + ["-o", LIB_PATH], verbose)
+    for o in objs:
+        os.remove(o)
     return LIB_PATH

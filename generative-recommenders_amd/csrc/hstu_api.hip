@@ -270,6 +270,12 @@ int current_device_cus() {
 
 }  // namespace
 
+// for the library's other translation units; not exported
+extern "C" __attribute__((visibility("hidden"))) int hstu_hip_device_is_gfx950(void) { return current_device_is_gfx950(); }
+extern "C" __attribute__((visibility("hidden"))) void hstu_hip_set_last_error(const char* what, int hip_error) {
+    set_last_error(what, (hipError_t)hip_error);
+}
+
 extern "C" {
 
 int hstu_hip_version(void) { return 100; }

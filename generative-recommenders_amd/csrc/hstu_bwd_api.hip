@@ -1,0 +1,133 @@
+// C ABI of the backward pass (hstu_hip_mha_bwd): validation and launch of the two kernels of hstu_bwd_kernel.h.
+// A translation unit of its own so that it compiles in parallel with the forward kernels.
+#include "hstu_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "hstu_bwd_kernel.h"
+
+// defined with the forward entry points (hstu_api.hip); internal to the library
+extern "C" __attribute__((visibility("hidden"))) int hstu_hip_device_is_gfx950(void);
+extern "C" __attribute__((visibility("hidden"))) void hstu_hip_set_last_error(const char* what, int hip_error);
+
+namespace {
+
+constexpr int kBwdWaves = 4, kBwdTile = 64, kBwdRows = kBwdWaves * 32;
+
+template <class TT, int DQK, int DV>
+int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
+    constexpr int smem = 2 * kBwdTile * (DQK + DV) * 2 + 64;  // + 64: transposing reads of a 16-wide tile's unused half
+    auto k1 = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
+    auto k2 = hstu::hstu_bwd_dq_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) {
+            hstu_hip_set_last_error("hipFuncSetAttribute", (int)e);
+            return HSTU_ERR_LAUNCH;
+        }
+        attr_done = true;
+    }
+    const unsigned grid = (unsigned)bp.f.slots_per_xcd * 8;
+    hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
+    hipLaunchKernelGGL(k2, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        hstu_hip_set_last_error("backward kernel launch", (int)e);
+        return HSTU_ERR_LAUNCH;
+    }
+    return HSTU_OK;
+}
+
+template <class TT, int DQK>
+int launch_bwd_dv(const hstu::BwdParams& bp, int dv, hipStream_t stream) {
+    switch (dv) {
+        case 16: return launch_bwd<TT, DQK, 16>(bp, stream);
+        case 32: return launch_bwd<TT, DQK, 32>(bp, stream);
+        case 64: return launch_bwd<TT, DQK, 64>(bp, stream);
+        case 128: return launch_bwd<TT, DQK, 128>(bp, stream);
+        default: return HSTU_ERR_BAD_HEAD_DIM;
+    }
+}
+
+template <class TT>
+int launch_bwd_dim(const hstu::BwdParams& bp, int dqk, int dv, hipStream_t stream) {
+    switch (dqk) {
+        case 16: return launch_bwd_dv<TT, 16>(bp, dv, stream);
+        case 32: return launch_bwd_dv<TT, 32>(bp, dv, stream);
+        case 64: return launch_bwd_dv<TT, 64>(bp, dv, stream);
+        case 128: return launch_bwd_dv<TT, 128>(bp, dv, stream);
+        default: return HSTU_ERR_BAD_HEAD_DIM;
+    }
+}
+
+}  // namespace
+
+extern "C" int hstu_hip_mha_bwd(const HstuFwdArgs* a, const HstuBwdGrads* g, void* stream_) {
+    if (!a || !g) return HSTU_ERR_NULL_POINTER;
+    HstuFwdArgs c = *a;  // the forward's own checks, with the unused output standing in as any aligned pointer
+    c.out = const_cast<void*>(a->q);
+    c.o_row_stride = c.o_head_stride = 0;
+    c.tile_config = 0;
+    c.kv_splits = 0;
+    int rc = hstu_hip_check_args(&c);
+    if (rc != HSTU_OK) return rc;
+    if (a->delta_size != 0) return HSTU_ERR_UNSUPPORTED;
+    if (a->dtype != HSTU_BF16 && a->dtype != HSTU_FP16) return HSTU_ERR_UNSUPPORTED;
+    if (a->total_q == 0 || a->batch == 0) return HSTU_OK;
+    if (!g->dout || !g->dq || !g->dk || !g->dv) return HSTU_ERR_NULL_POINTER;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(g->dout) | reinterpret_cast<uintptr_t>(g->dq) |
+                           reinterpret_cast<uintptr_t>(g->dk) | reinterpret_cast<uintptr_t>(g->dv);
+    if ((ptrs & 15) != 0) return HSTU_ERR_MISALIGNED;
+    const int64_t strides[8] = {g->do_row_stride, g->do_head_stride, g->dq_row_stride, g->dq_head_stride,
+                                g->dk_row_stride, g->dk_head_stride, g->dv_row_stride, g->dv_head_stride};
+    for (int i = 0; i < 8; ++i)
+        if (strides[i] < 0 || (strides[i] & 7) != 0) return HSTU_ERR_MISALIGNED;
+    if (!hstu_hip_device_is_gfx950()) return HSTU_ERR_BAD_DEVICE;
+    hipStream_t stream = (hipStream_t)stream_;
+
+    hstu::BwdParams bp;
+    memset(&bp, 0, sizeof(bp));
+    hstu::FwdParams& p = bp.f;
+    p.q = (const char*)a->q;
+    p.k = (const char*)a->k;
+    p.v = (const char*)a->v;
+    p.q_rs = a->q_row_stride, p.q_hs = a->q_head_stride;
+    p.k_rs = a->k_row_stride, p.k_hs = a->k_head_stride;
+    p.v_rs = a->v_row_stride, p.v_hs = a->v_head_stride;
+    p.offsets = a->seq_offsets;
+    p.targets = a->num_targets;
+    p.offsets_i64 = a->seq_offsets_i64;
+    p.targets_i64 = a->num_targets_i64;
+    p.B = a->batch;
+    p.H = a->heads;
+    p.max_seq_len = a->max_seq_len;
+    p.w = a->max_attn_len;
+    p.c = a->contextual_seq_len;
+    p.f = a->min_full_attn_seq_len;
+    p.kv_splits = 1;
+    p.c1 = -a->alpha * 1.4426950408889634f;
+    bp.gscale = a->alpha / (float)a->max_seq_len;
+    bp.pscale = a->alpha == 0.0f ? 0.0f : -1.0f / ((float)a->max_seq_len * 1.4426950408889634f);
+    bp.dout = (const char*)g->dout;
+    bp.dq = (char*)g->dq, bp.dk = (char*)g->dk, bp.dv = (char*)g->dv;
+    bp.do_rs = g->do_row_stride, bp.do_hs = g->do_head_stride;
+    bp.dq_rs = g->dq_row_stride, bp.dq_hs = g->dq_head_stride;
+    bp.dk_rs = g->dk_row_stride, bp.dk_hs = g->dk_head_stride;
+    bp.dv_rs = g->dv_row_stride, bp.dv_hs = g->dv_head_stride;
+
+    p.num_mb = (a->max_seq_len + kBwdRows - 1) / kBwdRows;
+    const long long pairs_per_xcd = ((long long)a->batch * a->heads + 7) / 8;
+    const long long slots = pairs_per_xcd * p.num_mb;
+    if (slots * 8 > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
+    p.pairs_per_xcd = (int)pairs_per_xcd;
+    p.slots_per_xcd = (int)slots;
+
+    // `sort_by_length` is a scheduling hint only; the backward kernels take the sequences in batch order
+    if (a->dtype == HSTU_BF16) return launch_bwd_dim<hstu::Bf16>(bp, a->dqk, a->dv, stream);
+    return launch_bwd_dim<hstu::Fp16>(bp, a->dqk, a->dv, stream);
+}

@@ -402,7 +402,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 // items, items of one class and pair stay neighbours (they share K/V through the L2), and row blocks past the
 // end of short sequences never become items.  A stable counting sort: the candidate items in pair-major order
 // are cut into 256 equal runs, one per thread; count per thread and class, scan over the threads, place.
-__global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(const FwdParams p, int bm, int bn, int* nitems, int* items) {
+static __global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(const FwdParams p, int bm, int bn, int* nitems, int* items) {
     constexpr int NC = 12;    // classes: up to 2^11 = 2048 tiles and more
     constexpr int NT = HSTU_PLAN_THREADS, NW = NT / 64;
     constexpr int CACHE = 32768;  // candidates whose class is remembered between the two walks
@@ -689,7 +689,7 @@ __device__ __forceinline__ void store_output(const f32x16_t (&oacc)[DT][QT], int
 }
 
 // dst[row][h][0..d) (dense, fp16) = src[row * rs + h * hs + 0..d) (fp32, strides in elements); 8 elements per thread.
-__global__ __launch_bounds__(256) void hstu_cast_f32_f16_kernel(const float* src, int64_t rs, int64_t hs, int64_t rows, int H,
+static __global__ __launch_bounds__(256) void hstu_cast_f32_f16_kernel(const float* src, int64_t rs, int64_t hs, int64_t rows, int H,
                                                                 int d, _Float16* dst) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // over rows * H * d / 8
     const int d8 = d >> 3;

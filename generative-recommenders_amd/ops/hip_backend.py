@@ -55,6 +55,25 @@ class HstuFwdArgs(ctypes.Structure):
     ]
 
 
+class HstuBwdGrads(ctypes.Structure):
+    """Mirror of ``HstuBwdGrads`` in include/hstu_hip.h (field order and types must match)."""
+
+    _fields_ = [
+        ("dout", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p),
+        ("dk", ctypes.c_void_p),
+        ("dv", ctypes.c_void_p),
+        ("do_row_stride", ctypes.c_int64),
+        ("do_head_stride", ctypes.c_int64),
+        ("dq_row_stride", ctypes.c_int64),
+        ("dq_head_stride", ctypes.c_int64),
+        ("dk_row_stride", ctypes.c_int64),
+        ("dk_head_stride", ctypes.c_int64),
+        ("dv_row_stride", ctypes.c_int64),
+        ("dv_head_stride", ctypes.c_int64),
+    ]
+
+
 class HstuJaggedCopyArgs(ctypes.Structure):
     """Mirror of ``HstuJaggedCopyArgs`` in include/hstu_hip.h (field order and types must match)."""
 
@@ -84,6 +103,7 @@ EXPORTS = (
     "hstu_hip_last_error",
     "hstu_hip_check_args",
     "hstu_hip_mha_fwd",
+    "hstu_hip_mha_bwd",
     "hstu_hip_workspace_bytes",
     "hstu_hip_plan",
     "hstu_hip_tile_configs",
@@ -118,6 +138,8 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_check_args.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_mha_fwd.restype = ctypes.c_int
         L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
+        L.hstu_hip_mha_bwd.restype = ctypes.c_int
+        L.hstu_hip_mha_bwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(HstuBwdGrads), ctypes.c_void_p]
         L.hstu_hip_plan.restype = ctypes.c_int
         L.hstu_hip_plan.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
         L.hstu_hip_workspace_bytes.restype = ctypes.c_size_t
@@ -266,6 +288,54 @@ def mha_fwd(
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
         rc = lib().hstu_hip_mha_fwd(ctypes.byref(a), ctypes.c_void_p(stream))
+    raise_for_status(rc)
+
+
+def mha_bwd(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    dq: torch.Tensor,
+    dk: torch.Tensor,
+    dv: torch.Tensor,
+    seq_offsets: torch.Tensor,
+    num_targets: Optional[torch.Tensor],
+    max_seq_len: int,
+    alpha: float,
+    max_attn_len: int,
+    contextual_seq_len: int,
+    min_full_attn_seq_len: int,
+) -> None:
+    """Fill ``dq``, ``dk``, ``dv`` on the current stream of ``q.device`` (full attention only)."""
+    a = HstuFwdArgs()
+    a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), None
+    a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
+    a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
+    a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
+    a.seq_offsets = seq_offsets.data_ptr()
+    a.seq_offsets_i64 = 1 if seq_offsets.dtype == torch.int64 else 0
+    if num_targets is not None:
+        a.num_targets = num_targets.data_ptr()
+        a.num_targets_i64 = 1 if num_targets.dtype == torch.int64 else 0
+    else:
+        a.num_targets = None
+    a.batch = seq_offsets.numel() - 1
+    a.heads, a.dqk, a.dv = q.shape[1], q.shape[2], v.shape[2]
+    a.total_q, a.total_kv = q.shape[0], k.shape[0]
+    a.max_seq_len, a.delta_size, a.alpha = max_seq_len, 0, alpha
+    a.max_attn_len, a.contextual_seq_len, a.min_full_attn_seq_len = max_attn_len, contextual_seq_len, min_full_attn_seq_len
+    a.dtype = _dtype_code(q.dtype)
+    a.q_scale = a.k_scale = a.v_scale = 1.0
+    g = HstuBwdGrads()
+    g.dout, g.dq, g.dk, g.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    g.do_row_stride, g.do_head_stride = dout.stride(0), dout.stride(1)
+    g.dq_row_stride, g.dq_head_stride = dq.stride(0), dq.stride(1)
+    g.dk_row_stride, g.dk_head_stride = dk.stride(0), dk.stride(1)
+    g.dv_row_stride, g.dv_head_stride = dv.stride(0), dv.stride(1)
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        rc = lib().hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), ctypes.c_void_p(stream))
     raise_for_status(rc)
 
 

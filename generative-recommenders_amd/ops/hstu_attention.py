@@ -6,7 +6,10 @@ messages and output shapes.  Differences, all explicit:
 
 * there is one backend, so ``kernel`` / ``enable_tma`` are accepted and ignored; ``sort_by_length`` is, as in
   the reference, a scheduling hint (long sequences are started first) that never changes the result;
-* forward only -- inputs that require grad under ``torch.enable_grad()`` raise ``NotImplementedError``;
+* ``hstu_mha`` is differentiable for bf16 / fp16 inputs (``dq, dk, dv`` come from the backward kernels through an
+  autograd function, as ``_AttentionFunction`` does in the reference, ``triton_hstu_attention.py:2978-3093``);
+  ``delta_hstu_mha`` and the fp32 / fp8 forms are forward only -- inputs that require grad under
+  ``torch.enable_grad()`` raise ``NotImplementedError`` there;
 * tensors must live on a HIP device; there is no CPU or PyTorch fallback;
 * fp32 q/k/v are rounded to fp16 inside the library (11-bit significand; the reference's Triton path multiplies in
   tf32) and give an fp32 result;
@@ -46,6 +49,41 @@ def _check_forward_only(*tensors: torch.Tensor) -> None:
             "the HIP backend implements the forward pass only; call it under torch.no_grad() "
             "or detach the inputs"
         )
+
+
+class _HstuMhaFunction(torch.autograd.Function):
+    """Forward and backward through the C ABI; saves only the inputs (the backward recomputes the scores)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
+                min_full_attn_seq_len, sort_by_length, tile_config, kv_splits):
+        q, k, v = _kernel_layout(q.detach()), _kernel_layout(k.detach()), _kernel_layout(v.detach())
+        out = torch.empty((v.shape[0], v.shape[1], v.shape[2]), dtype=v.dtype, device=v.device)
+        if out.numel() > 0:
+            hip_backend.mha_fwd(
+                q, k, v, out, seq_offsets, num_targets, max_seq_len=max_seq_len, alpha=alpha, delta_size=0,
+                max_attn_len=max_attn_len, contextual_seq_len=contextual_seq_len, min_full_attn_seq_len=min_full_attn_seq_len,
+                tile_config=tile_config, sort_by_length=sort_by_length, kv_splits=kv_splits,
+            )
+        ctx.save_for_backward(q, k, v, seq_offsets, *([] if num_targets is None else [num_targets]))
+        ctx.has_targets = num_targets is not None
+        ctx.params = (max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, seq_offsets = ctx.saved_tensors[:4]
+        num_targets = ctx.saved_tensors[4] if ctx.has_targets else None
+        max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len = ctx.params
+        # rows of sequences longer than max_seq_len are outside the contract and get no gradient
+        dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+        if q.numel() > 0:
+            dout = _kernel_layout(dout.detach())
+            hip_backend.mha_bwd(
+                dout, q, k, v, dq, dk, dv, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
+                min_full_attn_seq_len,
+            )
+        return (dq, dk, dv) + (None,) * 10
 
 
 def _require_device(t: torch.Tensor, name: str) -> None:
@@ -99,8 +137,14 @@ def hstu_mha(
         _require_device(num_targets, "num_targets")
         torch._assert(num_targets.numel() == seq_offsets.numel() - 1, "num_targets must have one entry per sequence")
         num_targets = _index_tensor(num_targets, "num_targets")
-    _check_forward_only(q, k, v)
     seq_offsets = _index_tensor(seq_offsets, "seq_offsets")
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+        if q.dtype not in (torch.bfloat16, torch.float16):
+            _check_forward_only(q, k, v)
+        return _HstuMhaFunction.apply(
+            q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len,
+            sort_by_length, tile_config, kv_splits,
+        )
 
     q = _kernel_layout(q.detach())
     k = _kernel_layout(k.detach())

@@ -135,6 +135,31 @@ int hstu_hip_tile_configs(void);
 const char* hstu_hip_tile_config_name(int id);
 
 /*
+ * ---- Backward of the full (non-delta) form ----
+ *
+ * dq, dk, dv from dout for the call described by `args` (its `out`, `tile_config`, `kv_splits` are ignored;
+ * `delta_size` must be 0; bf16 or fp16).  Replaces triton_hstu_attention_bwd
+ * (ops/triton/triton_hstu_attention.py:2825-2932, called from _AttentionFunction.backward, :3031-3093) and the
+ * native hstu_mha_bwd (ops/cpp/hstu_attention/flash_common.cpp:726 onwards).  Nothing from the forward call is
+ * needed except its inputs: the scores are recomputed.  Every row of dq / dk / dv that belongs to a sequence is
+ * written; no atomics, so the result is bit-identical from run to run.  The gradients have the layout rules of
+ * q / k / v: 16-byte aligned base, row and head strides in elements and multiples of 8, innermost stride 1.
+ * No workspace is used; `sort_by_length` (a scheduling hint) is ignored.
+ */
+typedef struct HstuBwdGrads {
+    const void* dout;  /* [total_q, H, dv] */
+    void* dq;          /* [total_q, H, dqk] */
+    void* dk;          /* [total_kv, H, dqk] */
+    void* dv;          /* [total_kv, H, dv] */
+    int64_t do_row_stride, do_head_stride;
+    int64_t dq_row_stride, dq_head_stride;
+    int64_t dk_row_stride, dk_head_stride;
+    int64_t dv_row_stride, dv_head_stride;
+} HstuBwdGrads;
+
+int hstu_hip_mha_bwd(const HstuFwdArgs* args, const HstuBwdGrads* grads, void* stream);
+
+/*
  * ---- The data format either side of the path: per-batch concatenation of two jagged 2-D tensors ----
  *
  * `left`, `right` and `joined` are row-major [rows, row_bytes] byte matrices with row strides in BYTES; batch b owns

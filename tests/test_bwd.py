@@ -1,0 +1,226 @@
+"""Backward of hstu_mha: the two CPU statements of the gradients against each other and against finite differences,
+then the HIP kernels against the closed form on the GPU.  Tolerance for bf16 / fp16 gradients (P and dS are rounded
+to the operand type before their products, as in the reference's kernel; fp32 accumulation): relative Frobenius
+error <= 1e-2 and max-abs error <= 2e-2 * max|ref| per gradient, against the fp32 closed form on the same (rounded)
+inputs."""
+
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import bwd_oracle as G
+from oracle import hstu_oracle as O
+
+
+def _inputs(seed, lengths, H, dqk, dv, dtype, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    offsets = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int64)
+    L = int(offsets[-1])
+    q = (torch.randn((L, H, dqk), generator=g) * scale).to(dtype)
+    k = (torch.randn((L, H, dqk), generator=g) * scale).to(dtype)
+    v = (torch.randn((L, H, dv), generator=g) * scale).to(dtype)
+    dout = (torch.randn((L, H, dv), generator=g) * scale).to(dtype)
+    return q, k, v, dout, offsets
+
+
+MASKS = [
+    dict(),
+    dict(max_attn_len=5),
+    dict(contextual_seq_len=3),
+    dict(num_targets=True),
+    dict(num_targets=True, max_attn_len=4, contextual_seq_len=2),
+    dict(num_targets=True, max_attn_len=3, contextual_seq_len=2, min_full_attn_seq_len=4),
+]
+
+
+def _mask_kwargs(mask, lengths, seed):
+    kw = dict(mask)
+    if kw.pop("num_targets", False):
+        rng = np.random.default_rng(seed)
+        c = kw.get("contextual_seq_len", 0)
+        kw["num_targets"] = torch.tensor([int(rng.integers(0, max(1, n - c))) if n > c else 0 for n in lengths], dtype=torch.int64)
+    return kw
+
+
+# ---------------------------------------------------------------- CPU
+
+
+@pytest.mark.parametrize("mi", range(len(MASKS)))
+def test_closed_form_matches_autograd(mi):
+    lengths = [17, 0, 24, 9, 1]
+    q, k, v, dout, offsets = _inputs(mi, lengths, 2, 8, 16, torch.float64)
+    kw = _mask_kwargs(MASKS[mi], lengths, mi)
+    a = G.autograd_grads(24, 0.3, q, k, v, offsets, dout, **kw)
+    c = G.closed_form_grads(24, 0.3, q, k, v, offsets, dout, dtype=torch.float64, row_chunk=7, **kw)
+    for name, x, y in zip(("dq", "dk", "dv"), a, c):
+        assert torch.allclose(x, y, atol=1e-12), name
+
+
+def test_forward_oracle_passes_finite_differences():
+    lengths = [5, 3]
+    q, k, v, _, offsets = _inputs(7, lengths, 1, 4, 4, torch.float64)
+    tg = torch.tensor([1, 0])
+
+    def f(q_, k_, v_):
+        return O.pytorch_hstu_mha(6, 0.7, q_, k_, v_, offsets, num_targets=tg, max_attn_len=3, contextual_seq_len=1)
+
+    assert torch.autograd.gradcheck(f, tuple(t.requires_grad_() for t in (q, k, v)), eps=1e-6, atol=1e-6)
+
+
+def test_silu_slope():
+    x = torch.tensor([0.0, 40.0, -40.0, 1.3, -0.7], dtype=torch.float64)
+    s = G.silu_slope(x)
+    assert float(s[0]) == 0.5 and abs(float(s[1]) - 1) < 1e-12 and abs(float(s[2])) < 1e-12
+    h = 1e-6
+    fd = (torch.nn.functional.silu(x + h) - torch.nn.functional.silu(x - h)) / (2 * h)
+    assert torch.allclose(s, fd, atol=1e-8)
+
+
+def test_gradients_are_linear_in_dout():
+    lengths = [12, 7]
+    q, k, v, dout, offsets = _inputs(3, lengths, 2, 8, 8, torch.float64)
+    a = G.closed_form_grads(12, 0.5, q, k, v, offsets, dout, dtype=torch.float64)
+    b = G.closed_form_grads(12, 0.5, q, k, v, offsets, -2.5 * dout, dtype=torch.float64)
+    for x, y in zip(a, b):
+        assert torch.allclose(-2.5 * x, y, atol=1e-12)
+
+
+# ---------------------------------------------------------------- GPU
+
+
+@pytest.fixture(scope="module")
+def pkg():
+    import __graft_entry__
+
+    return __graft_entry__.load_package()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    return torch.device("cuda:0")
+
+
+def _close(got, ref, what):
+    got, ref = got.float().cpu(), ref.float()
+    assert got.shape == ref.shape, what
+    assert torch.isfinite(got).all(), what
+    denom = float(ref.norm())
+    if denom == 0.0:
+        assert float(got.abs().max()) == 0.0, what
+        return
+    rel = float((got - ref).norm()) / denom
+    worst = float((got - ref).abs().max()) / float(ref.abs().max())
+    assert rel <= 1e-2 and worst <= 2e-2, f"{what}: relative {rel:.3e}, max-abs / max|ref| {worst:.3e}"
+
+
+def _run_bwd(pkg, dev, N, alpha, q, k, v, dout, offsets, offsets_dtype=torch.int64, **kw):
+    dkw = {a: (b.to(dev) if torch.is_tensor(b) else b) for a, b in kw.items()}
+    qd, kd, vd = (t.to(dev).requires_grad_() for t in (q, k, v))
+    out = pkg.hstu_mha(N, alpha, qd, kd, vd, offsets.to(offsets_dtype).to(dev), **dkw)
+    out.backward(dout.to(dev))
+    torch.cuda.synchronize()
+    return out.detach(), qd.grad, kd.grad, vd.grad
+
+
+def _check(pkg, dev, N, alpha, q, k, v, dout, offsets, what, **kw):
+    out, dq, dk, dv = _run_bwd(pkg, dev, N, alpha, q, k, v, dout, offsets, **kw)
+    rq, rk, rv = G.closed_form_grads(N, alpha, q, k, v, offsets, dout, **kw)
+    _close(dq, rq, what + " dq")
+    _close(dk, rk, what + " dk")
+    _close(dv, rv, what + " dv")
+    return dq, dk, dv
+
+
+GRID = [
+    # B, N, H, dqk, dv, mask index
+    (4, 200, 2, 64, 64, 0), (3, 300, 1, 128, 128, 0), (5, 130, 2, 32, 32, 1), (4, 257, 2, 128, 128, 4), (3, 200, 4, 64, 128, 3),
+    (2, 150, 2, 16, 16, 0), (3, 180, 1, 128, 32, 5), (4, 100, 3, 16, 64, 2), (2, 520, 2, 128, 128, 1), (6, 64, 2, 32, 128, 4),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,N,H,dqk,dv,mi", GRID)
+def test_backward_grid(pkg, dev, B, N, H, dqk, dv, mi, dtype):
+    print(f"[case] bwd grid {B} {N} {H} {dqk} {dv} mask={mi} {dtype}", flush=True)
+    rng = np.random.default_rng(B * 1000 + N)
+    lengths = [int(x) for x in rng.integers(1, N + 1, size=B)]
+    lengths[0] = N
+    q, k, v, dout, offsets = _inputs(N + dqk, lengths, H, dqk, dv, dtype)
+    scale = {0: 1.0, 5: 4.0}.get(mi, 20.0)  # windows and targets in proportion to these lengths
+    mask = {a: (int(b * scale) if isinstance(b, int) and not isinstance(b, bool) else b) for a, b in MASKS[mi].items()}
+    kw = _mask_kwargs(mask, lengths, N)
+    _check(pkg, dev, N, 1.0 / dqk**0.5, q, k, v, dout, offsets, "grid", **kw)
+
+
+EDGE = [
+    ([1], {}), ([2, 1, 3], {}), ([128], {}), ([129], {}), ([127, 64, 65, 63], {}), ([0, 40, 0], {}), ([256, 255, 257], {}),
+    ([300], dict(max_attn_len=1)), ([300], dict(max_attn_len=64)), ([300], dict(max_attn_len=1000)),
+    ([200, 90], dict(contextual_seq_len=70)), ([200, 140], dict(contextual_seq_len=130, max_attn_len=10)),
+    ([150, 150], dict(num_targets=torch.tensor([150, 0]))), ([150, 150], dict(num_targets=torch.tensor([149, 1]), max_attn_len=20)),
+    ([400], dict(num_targets=torch.tensor([100]), max_attn_len=50, contextual_seq_len=10, min_full_attn_seq_len=30)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("ei", range(len(EDGE)))
+def test_backward_edges(pkg, dev, ei):
+    lengths, kw = EDGE[ei]
+    print(f"[case] bwd edge {ei} {lengths}", flush=True)
+    q, k, v, dout, offsets = _inputs(ei, lengths, 2, 64, 64, torch.bfloat16)
+    _check(pkg, dev, max(lengths) + 3, 0.125, q, k, v, dout, offsets, f"edge {ei}", **kw)
+
+
+@pytest.mark.gpu
+def test_backward_is_deterministic_and_takes_views(pkg, dev):
+    print("[case] bwd determinism / strided views", flush=True)
+    lengths = [500, 300, 77]
+    q, k, v, dout, offsets = _inputs(21, lengths, 2, 128, 128, torch.bfloat16)
+    a = _run_bwd(pkg, dev, 512, 0.09, q, k, v, dout, offsets, offsets_dtype=torch.int32)
+    b = _run_bwd(pkg, dev, 512, 0.09, q, k, v, dout, offsets)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    # q, k, v as column slices of one buffer (the layout hstu_compute_uqvk returns); gradients identical
+    fused = torch.cat([q, k, v], dim=2).to(dev)
+    qs, ks, vs = (fused[:, :, i * 128 : (i + 1) * 128].detach().requires_grad_() for i in range(3))
+    out = pkg.hstu_mha(512, 0.09, qs, ks, vs, offsets.to(dev))
+    out.backward(dout.to(dev))
+    torch.cuda.synchronize()
+    for x, y in zip((qs.grad, ks.grad, vs.grad), b[1:]):
+        assert torch.equal(x, y)
+    assert torch.equal(out.detach(), b[0])
+
+
+@pytest.mark.gpu
+def test_backward_of_a_long_sequence(pkg, dev):
+    """4096 rows: 32 key blocks x 64 query tiles per pair, the shape the bench workload has per sequence."""
+    print("[case] bwd long", flush=True)
+    lengths = [4096, 1000]
+    q, k, v, dout, offsets = _inputs(5, lengths, 1, 128, 128, torch.bfloat16, scale=0.5)
+    _check(pkg, dev, 4096, 1.0 / 128**0.5, q, k, v, dout, offsets, "long")
+    kw = dict(num_targets=torch.tensor([300, 10]), max_attn_len=512, contextual_seq_len=6)
+    _check(pkg, dev, 4096, 1.0 / 128**0.5, q, k, v, dout, offsets, "long masked", **kw)
+
+
+@pytest.mark.gpu
+def test_backward_rejections(pkg, dev):
+    q, k, v, dout, offsets = _inputs(1, [40, 24], 2, 32, 32, torch.float32)
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_mha(64, 0.2, q.to(dev).requires_grad_(), k.to(dev), v.to(dev), offsets.to(dev))
+    with pytest.raises(NotImplementedError):
+        pkg.delta_hstu_mha(64, 0.2, q.bfloat16()[:16].to(dev).requires_grad_(), k.bfloat16().to(dev), v.bfloat16().to(dev), offsets.to(dev))
+    # no gradient asked for: the plain forward path, no graph
+    out = pkg.hstu_mha(64, 0.2, q.bfloat16().to(dev), k.bfloat16().to(dev), v.bfloat16().to(dev), offsets.to(dev))
+    assert not out.requires_grad
+    # only v requires grad: dq and dk are still produced and simply dropped by autograd
+    vd = v.bfloat16().to(dev).requires_grad_()
+    out = pkg.hstu_mha(64, 0.2, q.bfloat16().to(dev), k.bfloat16().to(dev), vd, offsets.to(dev))
+    out.sum().backward()
+    assert vd.grad is not None and torch.isfinite(vd.grad).all()
+    empty = pkg.hstu_mha(64, 0.2, q.bfloat16()[:0].to(dev).requires_grad_(), k.bfloat16()[:0].to(dev), v.bfloat16()[:0].to(dev),
+                         torch.zeros(1, dtype=torch.int64, device=dev))
+    assert empty.shape == (0, 2, 32)

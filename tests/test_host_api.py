@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol(backend):
     assert backend.tile_config_names() == ["m128n64w4", "m256n64w8pp", "m128n64w4pl"]
 
 
-@pytest.mark.parametrize("struct", ["HstuFwdArgs", "HstuJaggedCopyArgs"])
+@pytest.mark.parametrize("struct", ["HstuFwdArgs", "HstuJaggedCopyArgs", "HstuBwdGrads"])
 def test_struct_mirror_has_the_header_fields_in_order(backend, struct):
     header = open(os.path.join(ROOT, "include", "hstu_hip.h")).read()
     body = header[header.index(f"typedef struct {struct} {{") : header.index(f"}} {struct};")]
@@ -51,6 +51,28 @@ def test_struct_mirror_has_the_header_fields_in_order(backend, struct):
         names.append(re.findall(r"(\w+)\s*$", parts[0].strip())[0])
         names += [p.strip() for p in parts[1:]]
     assert names == [f[0] for f in getattr(backend, struct)._fields_]
+
+
+def test_backward_argument_checks(backend):
+    """Validation of hstu_hip_mha_bwd runs before anything touches the device."""
+    L = backend.lib()
+    a, g = backend.HstuFwdArgs(), backend.HstuBwdGrads()
+    assert L.hstu_hip_mha_bwd(None, ctypes.byref(g), None) == -1
+    assert L.hstu_hip_mha_bwd(ctypes.byref(a), None, None) == -1
+    a.batch, a.heads, a.dqk, a.dv, a.total_q, a.total_kv, a.max_seq_len, a.dtype = 2, 2, 64, 64, 0, 0, 16, 0
+    assert L.hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == 0  # nothing to do
+    a.delta_size, a.total_q, a.total_kv = 4, 8, 32
+    a.q = a.k = a.v = a.seq_offsets = 4096  # never dereferenced: the call is refused first
+    a.q_row_stride = a.k_row_stride = a.v_row_stride = 128
+    a.q_head_stride = a.k_head_stride = a.v_head_stride = 64
+    assert L.hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == -6  # delta mode has no backward
+    a.delta_size, a.total_q, a.dtype = 0, 32, 2
+    assert L.hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == -6  # nor has fp8
+    a.dtype = 0
+    assert L.hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == -1  # gradient pointers missing
+    g.dout = g.dq = g.dk = g.dv = 4096
+    g.do_row_stride = 127
+    assert L.hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == -4
 
 
 def test_jagged_copy_argument_checks(backend):
