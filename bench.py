@@ -267,6 +267,76 @@ def run_linear(name, args, pkg, torch):
     print(json.dumps(line))
 
 
+def run_bwd(name, args, pkg, workloads, torch):
+    """Backward of hstu_mha (dq, dk, dv from dout) on the headline shape (`bwd`) or on the ragged third baseline
+    configuration (`bwd_cfg3`).  A step is one call of the backward entry point: its two kernels.  Algorithmic work:
+    five products per mask-valid pair (S, dP, dV, dQ, dK -- the count of the reference's bench,
+    ops/benchmarks/hstu_attention_bench.py:51-60), i.e. 2 * (3 * Dqk + 2 * Dv) flops."""
+    from generative_recommenders_amd.ops import hip_backend
+
+    from oracle import bwd_oracle
+
+    dev = torch.device("cuda:0")
+    wl = workloads.make_workload("headline" if name == "bwd" else "cfg3")
+    inp = workloads.make_inputs(wl, dev)
+    q, k, v, offsets, targets = inp["q"], inp["k"], inp["v"], inp["seq_offsets"], inp["num_targets"]
+    g = torch.Generator(device=dev).manual_seed(wl.seed + 1)
+    dout = (torch.randn(v.shape, device=dev, generator=g) * 0.1).to(v.dtype)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+    def step():
+        hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offsets, targets, wl.max_seq_len, wl.alpha, wl.max_attn_len,
+                            wl.contextual_seq_len, wl.min_full_attn_seq_len)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    wall_ms, ev_ms = timed_steps(step, args, torch, flush=False)
+    pair_flops = 2.0 * (3 * wl.dqk + 2 * wl.dv)
+    flops = workloads.algorithmic_flops(wl) / (2.0 * (wl.dqk + wl.dv)) * pair_flops
+    nbytes = 2.0 * wl.total_kv * wl.heads * (4 * wl.dqk + 3 * wl.dv)  # q, k, dq, dk and v, dout, dv once each
+    tflops = flops / (ev_ms * 1e-3) / 1e12
+    line = {
+        "metric": "HSTU attn bwd effective TFLOP/s + % MFMA peak", "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
+        "config": {"workload": name, "batch": wl.batch, "heads": wl.heads, "dqk": wl.dqk, "dv": wl.dv, "max_seq_len": wl.max_seq_len,
+                   "total_tokens": wl.total_kv, "max_attn_len": wl.max_attn_len, "contextual_seq_len": wl.contextual_seq_len,
+                   "num_targets": wl.num_targets is not None},
+        "pct_mfma_peak": round(100.0 * tflops / PEAK_TFLOPS[wl.dtype], 2),
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_TFLOPS[wl.dtype], "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_TFLOPS[wl.dtype], 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+                     "kernel": "hstu_bwd_dkdv_kernel + hstu_bwd_dq_kernel", "kernel_ms": round(ev_ms, 4),
+                     "algorithmic_flops": flops, "algorithmic_bytes": nbytes},
+    }
+    if not args.no_cpu:
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        order = sorted(range(wl.batch), key=lambda b: -int(wl.lengths[b]))
+        picks = [order[0]] + order[8::8]
+        qc, kc, vc, dc = [t.float().cpu() for t in (q, k, v, dout)]
+        oc, tc = offsets.cpu(), None if targets is None else targets.cpu()
+        done, cpu_flops, t_used = [], 0.0, 0.0
+        import numpy as np
+        for b in picks:
+            t0 = time.perf_counter()
+            bwd_oracle.closed_form_grads(wl.max_seq_len, wl.alpha, qc, kc, vc, oc, dc, num_targets=tc, max_attn_len=wl.max_attn_len,
+                                         contextual_seq_len=wl.contextual_seq_len, min_full_attn_seq_len=wl.min_full_attn_seq_len,
+                                         sequences=[b])
+            t_used += time.perf_counter() - t0
+            sub = workloads.Workload("s", 1, wl.heads, wl.dqk, wl.dv, wl.max_seq_len, np.asarray(wl.lengths[b : b + 1]),
+                                     None if wl.num_targets is None else np.asarray(wl.num_targets[b : b + 1]), wl.max_attn_len,
+                                     wl.contextual_seq_len, wl.min_full_attn_seq_len, 0, wl.dtype, wl.alpha, wl.seed)
+            cpu_flops += workloads.algorithmic_flops(sub) / (2.0 * (wl.dqk + wl.dv)) * pair_flops
+            done.append(b)
+            if t_used > 15.0:
+                break
+        line["cpu_baseline"] = {"value": round(cpu_flops / t_used / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                                "sample": f"{len(done)} of {wl.batch} sequences (lengths {[int(wl.lengths[b]) for b in done]}), "
+                                          f"fp32 closed-form gradients per sequence, {t_used:.1f} s"}
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -299,7 +369,8 @@ def main():
 
     jagged = args.workload in ("kvcat", "kvtail")
     producer = args.workload in ("uqvk", "layernorm", "output", "normmul")
-    wl = None if jagged or producer else workloads.make_workload(args.workload)
+    backward = args.workload in ("bwd", "bwd_cfg3")
+    wl = None if jagged or producer or backward else workloads.make_workload(args.workload)
     if wl is not None and wl.dtype == "fp32":
         print("bench.py: cfg1 is the CPU correctness case, not a GPU bench workload", file=sys.stderr)
         sys.exit(2)
@@ -315,6 +386,9 @@ def main():
         return
     if producer:
         run_linear(args.workload, args, pkg, torch)
+        return
+    if backward:
+        run_bwd(args.workload, args, pkg, workloads, torch)
         return
     wall_ms, ev_ms = run_gpu(wl, args, pkg, workloads, torch)
     flops = workloads.algorithmic_flops(wl)
