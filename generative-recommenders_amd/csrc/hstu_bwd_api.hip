@@ -19,12 +19,13 @@ constexpr int kBwdWaves = 4, kBwdTile = 64, kBwdRows = kBwdWaves * 32;
 
 template <class TT, int DQK, int DV>
 int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
-    constexpr int smem = 2 * kBwdTile * (DQK + DV) * 2 + 64;  // + 64: transposing reads of a 16-wide tile's unused half
+    // three tile slots for the key-stationary kernel, two for the other; + 64: transposing reads of a 16-wide tile's unused half
+    constexpr int smem1 = 3 * kBwdTile * (DQK + DV) * 2 + 64, smem = 2 * kBwdTile * (DQK + DV) * 2 + 64;
     auto k1 = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
     auto k2 = hstu::hstu_bwd_dq_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
     static bool attr_done = false;
     if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) {
             hstu_hip_set_last_error("hipFuncSetAttribute", (int)e);
@@ -33,7 +34,7 @@ int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
         attr_done = true;
     }
     const unsigned grid = (unsigned)bp.f.slots_per_xcd * 8;
-    hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
+    hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
     hipLaunchKernelGGL(k2, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {

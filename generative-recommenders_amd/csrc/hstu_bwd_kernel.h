@@ -26,6 +26,8 @@
 // A tile that is read both by rows (ds_read_b128) and transposed (ds_read_b64_tr_b16) is stored with one chunk
 // swizzle that keeps both kinds of read off each other's banks (swz_u below).
 #pragma once
+#include <type_traits>
+
 #include "hstu_common.h"
 
 namespace hstu {
@@ -165,15 +167,38 @@ struct KeyMask {
     }
 };
 
+// Order in which two chains of NA and NB accumulating MFMAs are issued: alternately while both last, so that
+// neighbours never depend on each other.
+template <int NA, int NB>
+struct TwoChains {
+    static constexpr int N = NA + NB;
+    static constexpr int M = NA < NB ? NA : NB;
+    static constexpr bool first(int k) { return k < 2 * M ? (k & 1) == 0 : NA > NB; }
+    static constexpr int index(int k) { return k < 2 * M ? k / 2 : k - M; }
+};
+
+// The key-stationary kernel has two 128-row accumulators and K, V in registers: one wave per SIMD.  A wave alone
+// must therefore overlap its own matrix and VALU work, which it does by software pipelining over blocks of 32
+// query rows: phase A issues the S and dP products of the NEXT block, one MFMA at a time, each followed by the
+// pointwise work (sigmoid, slope, mask, rounding) on one accumulator element of the CURRENT block; phase B then
+// issues the dV and dK products of the current block.  LDS operands are requested PD MFMAs ahead.  Tiles of 64
+// query rows sit in three LDS slots; the one barrier per tile comes after the first block of a tile has gone through
+// phase B, when nobody can still read the tile before it, whose slot the next copy overwrites.
+// Blocks are skipped per wave only in whole phases (a block with no valid pair for the wave's keys gets neither
+// products nor pointwise work); the barrier count per tile is the same for every wave.
 template <class TT, int DQK, int DV, int NW, int BN>
 __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdParams bp) {
     typedef typename TT::vec8 vec8;
+    static_assert(BN == 64, "two blocks of 32 query rows per tile");
     const FwdParams& p = bp.f;
     constexpr int BM = NW * 32;  // key rows per workgroup
     constexpr int KS = DQK / 16, VS = DV / 16, DTK = (DQK + 31) / 32, DTV = (DV + 31) / 32;
     constexpr int QROW = DQK * 2, OROW = DV * 2;
     constexpr int QTILE = BN * QROW, OTILE = BN * OROW, STAGE = QTILE + OTILE;
     constexpr int NT = NW * 64;
+    constexpr int PD = 3;  // LDS operands in flight ahead of the MFMA that uses them
+    typedef TwoChains<KS, VS> OpsA;
+    typedef TwoChains<2 * DTV, 2 * DTK> OpsB;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
 
     const int lane = threadIdx.x & 63;
@@ -187,7 +212,7 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
     const int S0 = W.R0, S1 = W.R1;  // key rows of the workgroup (inclusive)
     const int wS0 = S0 + wave * 32;  // first key row of the wave; the wave has no keys if wS0 > S1
 
-    // query tiles [jt, jt_end): rows at or after the first key (all rows if a contextual prefix sees every key), up
+    // query tiles [.., jt_end): rows at or after the first key (all rows if a contextual prefix sees every key), up
     // to the last row whose window still reaches the block (targets sit at id max_id)
     int q_hi = n - 1;
     if (M.w > 0 && M.f == 0) {
@@ -208,16 +233,19 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
             }
         return jt;
     };
-    int jt = next_tile(M.c > 0 ? 0 : S0 / BN);
 
     const char* qbase = p.q + (W.seq_start * p.q_rs + (int64_t)W.h * p.q_hs) * 2;
     const char* obase = bp.dout + (W.seq_start * bp.do_rs + (int64_t)W.h * bp.do_hs) * 2;
     const int64_t q_rsb = p.q_rs * 2, o_rsb = bp.do_rs * 2;
+    auto copy_tile = [&](int jt, int slot) {
+        load_tile_u<BN, QROW, NT>(qbase, q_rsb, jt * BN, n - 1, smem + slot * STAGE, wave, lane);
+        load_tile_u<BN, OROW, NT>(obase, o_rsb, jt * BN, n - 1, smem + slot * STAGE + QTILE, wave, lane);
+    };
 
-    if (jt < jt_end) {
-        load_tile_u<BN, QROW, NT>(qbase, q_rsb, jt * BN, n - 1, smem, wave, lane);
-        load_tile_u<BN, OROW, NT>(obase, o_rsb, jt * BN, n - 1, smem + QTILE, wave, lane);
-    }
+    int t_cur = next_tile(M.c > 0 ? 0 : S0 / BN);
+    int t_nxt = t_cur < jt_end ? next_tile(t_cur + 1) : jt_end;
+    if (t_cur < jt_end) copy_tile(t_cur, 0);
+    if (t_nxt < jt_end) copy_tile(t_nxt, 1);
 
     vec8 kreg[KS], vreg[VS];
     load_q_operand<TT, KS>(kreg, p.k, W.seq_start, wS0 + l32, n, p.k_rs, p.k_hs, W.h, g, p.c1);
@@ -238,68 +266,149 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
         for (int dt = 0; dt < DTV; ++dt) dvacc[dt][0][r] = 0.f;
     }
 
-    int stage = 0;
-    while (jt < jt_end) {
-        const int jn = next_tile(jt + 1);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this tile's copies have landed
-        __syncthreads();
-        if (jn < jt_end) {
-            char* nxt = smem + (stage ^ 1) * STAGE;
-            load_tile_u<BN, QROW, NT>(qbase, q_rsb, jn * BN, n - 1, nxt, wave, lane);
-            load_tile_u<BN, OROW, NT>(obase, o_rsb, jn * BN, n - 1, nxt + QTILE, wave, lane);
+    // class of the block of 32 query rows starting at r0 against this wave's keys: 0 nothing valid, 1 masked, 2 all valid
+    auto block_class = [&](int r0) {
+        if (r0 >= n || wS0 > S1) return 0;
+        const int r1 = r0 + 31 < n ? r0 + 31 : n - 1;
+        int cls = M.classify(r0, r1, wS0, 32);
+        if (cls == 2 && r0 + 31 >= n) cls = 1;
+        return cls;
+    };
+
+    // Phase A.  MFMA: issue S and dP of the block whose Q / dOut rows start at qn / on into (s_n, dp_n).
+    // PW (0 none, 1 masked, 2 all valid): P and dS of the block held in (s_c, dp_c), whose first query row is r0_c,
+    // packed into pb / dsb.
+    auto phase_a = [&](auto mfma_c, auto pw_c, const char* qn, const char* on, f32x16_t& s_n, f32x16_t& dp_n, const f32x16_t& s_c,
+                       const f32x16_t& dp_c, int r0_c, vec8 (&pb)[2], vec8 (&dsb)[2]) __attribute__((always_inline)) {
+        constexpr bool MFMA = decltype(mfma_c)::value;
+        constexpr int PW = decltype(pw_c)::value;
+        constexpr int NA = OpsA::N;
+        auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
+            return OpsA::first(k) ? *HSTU_LDS(const vec8, qn + qrow[OpsA::index(k)]) : *HSTU_LDS(const vec8, on + orow[OpsA::index(k)]);
+        };
+        vec8 fr[PD];
+        if constexpr (MFMA) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_n[r] = dp_n[r] = 0.f;
+#pragma unroll
+            for (int k = 0; k < PD && k < NA; ++k) fr[k] = load_op(k);
         }
-        const char* qt = smem + stage * STAGE;
-        const char* ot = qt + QTILE;
+        float pv[16], dsv[16];
 #pragma unroll
-        for (int sub = 0; sub < BN / 32; ++sub) {
-            const int r0 = jt * BN + sub * 32;  // first query row of the block of 32
-            if (r0 >= n || wS0 > S1) continue;
-            const int r1 = r0 + 31 < n ? r0 + 31 : n - 1;
-            int cls = M.classify(r0, r1, wS0, 32);
-            if (cls == 2 && r0 + 31 >= n) cls = 1;
-            if (cls == 0) continue;
-            f32x16_t s, dp;
+        for (int k = 0; k < NA; ++k) {
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (MFMA) {
+                if (OpsA::first(k)) s_n = TT::mfma(fr[k % PD], kreg[OpsA::index(k)], s_n);
+                else dp_n = TT::mfma(fr[k % PD], vreg[OpsA::index(k)], dp_n);
+                if (k + PD < NA) fr[k % PD] = load_op(k + PD);
+            }
+            if constexpr (PW != 0) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) s = TT::mfma(*HSTU_LDS(const vec8, qt + sub * 32 * QROW + qrow[ks]), kreg[ks], s);
-#pragma unroll
-            for (int ks = 0; ks < VS; ++ks) dp = TT::mfma(*HSTU_LDS(const vec8, ot + sub * 32 * OROW + orow[ks]), vreg[ks], dp);
-            vec8 pb[2], dsb[2];
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                float pv[8], dv8[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int r = half * 8 + j;
+                for (int e = 0; e < 16; ++e) {
+                    if (e * NA / 16 != k) continue;
                     float pr, gr;
-                    silu_and_slope(s[r], pr, gr);
-                    float dsr = dp[r] * gr;
-                    if (cls == 1) {
-                        const bool ok = key.valid(M, r0 + 8 * (r >> 2) + 4 * g + (r & 3));
+                    silu_and_slope(s_c[e], pr, gr);
+                    float dsr = dp_c[e] * gr;
+                    if constexpr (PW == 1) {
+                        const bool ok = key.valid(M, r0_c + 8 * (e >> 2) + 4 * g + (e & 3));
                         pr = ok ? pr : 0.f;
                         dsr = ok ? dsr : 0.f;
                     }
-                    pv[j] = pr;
-                    dv8[j] = dsr;
+                    pv[e] = pr;
+                    dsv[e] = dsr;
+                    if (e == 7 || e == 15) {
+                        float p8[8], d8[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            p8[j] = pv[e - 7 + j];
+                            d8[j] = dsv[e - 7 + j];
+                        }
+                        pb[e >> 3] = TT::pack8(p8);
+                        dsb[e >> 3] = TT::pack8(d8);
+                    }
                 }
-                pb[half] = TT::pack8(pv);
-                dsb[half] = TT::pack8(dv8);
-            }
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const char* ob = ot + (sub * 32 + tt * 16) * OROW;
-                const char* qb = qt + (sub * 32 + tt * 16) * QROW;
-#pragma unroll
-                for (int dt = 0; dt < DTV; ++dt)
-                    dvacc[dt][0] = TT::mfma(read_vt_operand<TT>(ob + otr[0][dt], ob + otr[1][dt]), pb[tt], dvacc[dt][0]);
-#pragma unroll
-                for (int dt = 0; dt < DTK; ++dt)
-                    dkacc[dt][0] = TT::mfma(read_vt_operand<TT>(qb + qtr[0][dt], qb + qtr[1][dt]), dsb[tt], dkacc[dt][0]);
             }
         }
-        jt = jn;
-        stage ^= 1;
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // Phase B: dV^T += dOut^T P and dK^T += Q^T dS for the block whose rows start at qc / oc.
+    auto phase_b = [&](const char* qc, const char* oc, const vec8 (&pb)[2], const vec8 (&dsb)[2]) __attribute__((always_inline)) {
+        constexpr int NB = OpsB::N;
+        auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
+            const int i = OpsB::index(k);
+            if (OpsB::first(k)) {
+                const char* b = oc + (i / DTV) * 16 * OROW;
+                return read_vt_operand<TT>(b + otr[0][i % DTV], b + otr[1][i % DTV]);
+            }
+            const char* b = qc + (i / DTK) * 16 * QROW;
+            return read_vt_operand<TT>(b + qtr[0][i % DTK], b + qtr[1][i % DTK]);
+        };
+        vec8 fr[PD];
+#pragma unroll
+        for (int k = 0; k < PD && k < NB; ++k) fr[k] = load_op(k);
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            __builtin_amdgcn_sched_barrier(0);
+            const int i = OpsB::index(k);
+            if (OpsB::first(k)) dvacc[i % DTV][0] = TT::mfma(fr[k % PD], pb[i / DTV], dvacc[i % DTV][0]);
+            else dkacc[i % DTK][0] = TT::mfma(fr[k % PD], dsb[i / DTK], dkacc[i % DTK][0]);
+            if (k + PD < NB) fr[k % PD] = load_op(k + PD);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    typedef std::integral_constant<bool, true> Yes;
+    typedef std::integral_constant<bool, false> No;
+    typedef std::integral_constant<int, 0> Pw0;
+    typedef std::integral_constant<int, 1> Pw1;
+    typedef std::integral_constant<int, 2> Pw2;
+    // phase A with the two choices made at run time (both are wave-uniform)
+    auto run_a = [&](bool mfma, int pw, const char* qn, const char* on, f32x16_t& s_n, f32x16_t& dp_n, const f32x16_t& s_c,
+                     const f32x16_t& dp_c, int r0_c, vec8 (&pb)[2], vec8 (&dsb)[2]) __attribute__((always_inline)) {
+        if (mfma) {
+            if (pw == 2) phase_a(Yes{}, Pw2{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
+            else if (pw == 1) phase_a(Yes{}, Pw1{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
+            else phase_a(Yes{}, Pw0{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
+        } else {
+            if (pw == 2) phase_a(No{}, Pw2{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
+            else if (pw == 1) phase_a(No{}, Pw1{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
+        }
+    };
+
+    if (t_cur < jt_end) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first tiles have landed
+        __syncthreads();
+        f32x16_t sx, dpx, sy, dpy;  // block 0 of a tile lives in x, block 1 in y
+        vec8 pb[2], dsb[2];
+        int slot = 0;
+        int clsx = block_class(t_cur * BN);
+        run_a(clsx != 0, 0, smem, smem + QTILE, sx, dpx, sx, dpx, 0, pb, dsb);
+        while (true) {
+            const char* qt = smem + slot * STAGE;
+            const char* ot = qt + QTILE;
+            // block 1 of this tile enters phase A while block 0 gets its pointwise work
+            const int clsy = block_class(t_cur * BN + 32);
+            run_a(clsy != 0, clsx, qt + 32 * QROW, ot + 32 * OROW, sy, dpy, sx, dpx, t_cur * BN, pb, dsb);
+            if (clsx != 0) phase_b(qt, ot, pb, dsb);
+            const bool more = t_nxt < jt_end;
+            int t_nn = jt_end;
+            if (more) {
+                __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile, copied during the last one, has landed
+                __syncthreads();                      // ... for every wave; and nobody reads the tile before this one any more
+                t_nn = next_tile(t_nxt + 1);
+                const int nslot = slot == 2 ? 0 : slot + 1;
+                if (t_nn < jt_end) copy_tile(t_nn, nslot == 2 ? 0 : nslot + 1);
+                clsx = block_class(t_nxt * BN);
+                const char* qn = smem + nslot * STAGE;
+                run_a(clsx != 0, clsy, qn, qn + QTILE, sx, dpx, sy, dpy, t_cur * BN + 32, pb, dsb);
+            } else {
+                run_a(false, clsy, qt, ot, sx, dpx, sy, dpy, t_cur * BN + 32, pb, dsb);
+            }
+            if (clsy != 0) phase_b(qt + 32 * QROW, ot + 32 * OROW, pb, dsb);
+            if (!more) break;
+            t_cur = t_nxt;
+            t_nxt = t_nn;
+            slot = slot == 2 ? 0 : slot + 1;
+        }
     }
     store_output<TT, DTK>(dkacc, 0, bp.dk, W.seq_start, wS0 + l32, n, bp.dk_rs, bp.dk_hs, W.h, g, bp.gscale, DQK);
     store_output<TT, DTV>(dvacc, 0, bp.dv, W.seq_start, wS0 + l32, n, bp.dv_rs, bp.dv_hs, W.h, g, bp.pscale, DV);
