@@ -11,6 +11,8 @@
 #include <mutex>
 #include <tuple>
 
+#include "hstu_uqvk_kernel.h"
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -383,6 +385,46 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
     return 0;
 }
 
+bool uqvk_fused_shape(const HstuUqvkArgs* a) {
+    const int n_u = a->hidden_dim * a->heads;
+    const int n_out = (2 * a->hidden_dim + 2 * a->attn_dim) * a->heads;
+    return (a->d_model == 128 || a->d_model == 256 || a->d_model == 384 || a->d_model == 512) && n_u % 128 == 0 && n_out % 128 == 0 &&
+           (a->dtype == 0 || a->dtype == 1);
+}
+
+template <class TT, int KT>
+int launch_uqvk_fused(const hstu::UqvkFusedParams& p, hipStream_t stream) {
+    auto kern = hstu::hstu_uqvk_fused_kernel<TT, KT>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, hstu::kUqvkLds);
+        if (e != hipSuccess) {
+            snprintf(g_last_error, sizeof(g_last_error), "hipFuncSetAttribute: %s", hipGetErrorString(e));
+            return -7;
+        }
+        attr_done = true;
+    }
+    constexpr int kRows = hstu::kUqvkWaves * hstu::kUqvkRowsPerWave;
+    const long long grid = (p.rows + kRows - 1) / kRows;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(hstu::kUqvkWaves * 64), hstu::kUqvkLds, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        snprintf(g_last_error, sizeof(g_last_error), "fused uqvk kernel launch: %s", hipGetErrorString(e));
+        return -7;
+    }
+    return 0;
+}
+
+template <class TT>
+int launch_uqvk_fused_k(const hstu::UqvkFusedParams& p, int d_model, hipStream_t stream) {
+    switch (d_model) {
+        case 128: return launch_uqvk_fused<TT, 2>(p, stream);
+        case 256: return launch_uqvk_fused<TT, 4>(p, stream);
+        case 384: return launch_uqvk_fused<TT, 6>(p, stream);
+        default: return launch_uqvk_fused<TT, 8>(p, stream);
+    }
+}
+
 size_t normed_bytes(const HstuUqvkArgs* a) { return (((size_t)a->rows * a->d_model * 2) + 255) & ~(size_t)255; }
 size_t joined_bytes(const HstuOutputArgs* a) {
     return (((size_t)a->rows * output_blocks(a) * a->heads * a->linear_dim * 2) + 255) & ~(size_t)255;
@@ -396,6 +438,7 @@ const char* hstu_linear_last_error(void) { return g_last_error; }
 
 size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* a) {
     if (!a || a->rows <= 0 || a->d_model <= 0) return 0;
+    if (a->path != 1 && a->heads > 0 && a->attn_dim > 0 && a->hidden_dim > 0 && uqvk_fused_shape(a)) return 0;
     return normed_bytes(a) + kGemmScratch;
 }
 
@@ -410,13 +453,30 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
     if (!a) return -1;
     if (a->rows < 0 || a->heads <= 0 || a->attn_dim <= 0 || a->hidden_dim <= 0 || a->d_model <= 0) return -5;
     if (a->rows == 0) return 0;
-    if (!a->uvqk_weight || !a->uvqk_bias || !a->uvqk || !a->workspace) return -1;
-    if ((size_t)a->workspace_bytes < hstu_uqvk_workspace_bytes(a) || ((uintptr_t)a->workspace & 255) != 0) return -4;
+    if (a->path < 0 || a->path > 2) return -5;
+    if (!a->uvqk_weight || !a->uvqk_bias || !a->uvqk) return -1;
     if (a->rows > 0x7fffffffLL) return -5;
     hipStream_t stream = (hipStream_t)stream_;
     const int n_u = a->hidden_dim * a->heads;
     const int n_out = (2 * a->hidden_dim + 2 * a->attn_dim) * a->heads;
     if ((n_u & 7) != 0 || (n_out & 7) != 0) return -4;  // column blocks start on 16-byte boundaries
+    const bool fused = a->path != 1 && uqvk_fused_shape(a);
+    if (a->path == 2 && !fused) return -6;
+    if (fused) {
+        if (!a->x || !a->norm_weight || !a->norm_bias) return -1;
+        if (a->x_row_stride < a->d_model || (a->x_row_stride & 7) != 0) return -5;
+        const uintptr_t ptrs = (uintptr_t)a->x | (uintptr_t)a->norm_weight | (uintptr_t)a->norm_bias | (uintptr_t)a->uvqk_weight |
+                               (uintptr_t)a->uvqk_bias | (uintptr_t)a->uvqk;
+        if ((ptrs & 15) != 0) return -4;
+        hstu::UqvkFusedParams p;
+        p.x = (const char*)a->x, p.x_rs = a->x_row_stride;
+        p.norm_weight = (const char*)a->norm_weight, p.norm_bias = (const char*)a->norm_bias, p.eps = a->norm_eps;
+        p.w = (const char*)a->uvqk_weight, p.bias = (const char*)a->uvqk_bias, p.out = (char*)a->uvqk;
+        p.rows = a->rows, p.n_out = n_out, p.n_silu = n_u;
+        return a->dtype == 0 ? launch_uqvk_fused_k<hstu::Bf16>(p, a->d_model, stream) : launch_uqvk_fused_k<hstu::Fp16>(p, a->d_model, stream);
+    }
+    if (!a->workspace) return -1;
+    if ((size_t)a->workspace_bytes < hstu_uqvk_workspace_bytes(a) || ((uintptr_t)a->workspace & 255) != 0) return -4;
     void* normed = a->workspace;
     void* scratch = (char*)a->workspace + normed_bytes(a);
     int rc = launch_layer_norm(a->x, a->x_row_stride, a->norm_weight, a->norm_bias, a->norm_eps, normed, a->d_model, a->rows,

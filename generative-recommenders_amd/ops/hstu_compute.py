@@ -43,6 +43,7 @@ class HstuUqvkArgs(ctypes.Structure):
         ("dtype", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
+        ("path", ctypes.c_int32),
     ]
 
 
@@ -169,9 +170,11 @@ def hstu_compute_uqvk(
     uvqk_weight: torch.Tensor,
     uvqk_bias: torch.Tensor,
     kernel: HammerKernel = HammerKernel.HIP,
+    path: int = 0,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Returns ``(u, q, k, v)``: ``u [L, hidden*H]`` already through SiLU, ``q, k [L, H, attn]``, ``v [L, H, hidden]``,
-    all views of one buffer."""
+    all views of one buffer.  ``path``: 0 = the fused kernel where the shape allows, else layer-norm kernel +
+    hipBLASLt; 1 / 2 force one or the other."""
     torch._assert(x.dim() == 2, "x must be 2-D")
     n_out = (2 * hidden_dim + 2 * attn_dim) * num_heads
     torch._assert(uvqk_weight.shape == (x.shape[1], n_out), "uvqk_weight must be [d_model, (2*hidden + 2*attn) * heads]")
@@ -190,11 +193,12 @@ def hstu_compute_uqvk(
     a.rows, a.d_model = x.shape[0], x.shape[1]
     a.heads, a.attn_dim, a.hidden_dim = num_heads, attn_dim, hidden_dim
     a.dtype = _dtype_code(x.dtype)
+    a.path = path
     if x.shape[0] > 0:
         need = lib().hstu_uqvk_workspace_bytes(ctypes.byref(a))
-        workspace = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
-        base = (workspace.data_ptr() + 255) & ~255
-        a.workspace, a.workspace_bytes = base, need
+        if need > 0:
+            workspace = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
+            a.workspace, a.workspace_bytes = (workspace.data_ptr() + 255) & ~255, need
         with torch.cuda.device(x.device):
             stream = torch.cuda.current_stream(x.device).cuda_stream
             rc = lib().hstu_uqvk_forward(ctypes.byref(a), ctypes.c_void_p(stream))

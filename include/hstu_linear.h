@@ -10,9 +10,11 @@
  * All four results stay column slices of ONE [L, n_out] buffer -- the layout the attention entry points read in
  * place through their row / head strides -- so nothing is copied on the way to `hstu_hip_mha_fwd`.
  *
- * The layer norm is a hand-written kernel (one wave per row, HBM-bound).  The matrix product is a plain GEMM and
- * goes to hipBLASLt, with the bias and, for the u columns, the SiLU in the GEMM's epilogue.  This library is
- * separate from libhstu_hip.so so that the attention library does not depend on hipBLASLt.
+ * Two paths.  Fused (the usual shapes, see `path`): one hand-written kernel that keeps a wave's 32 normalised rows in
+ * registers as MFMA operands, streams the weight through LDS and applies bias and SiLU before the store -- x is read
+ * once, uvqk written once, nothing else touches HBM.  Library path (any shape): a layer-norm kernel (one wave per row)
+ * and hipBLASLt with the bias and, for the u columns, the SiLU in the GEMM's epilogue.  This library is separate from
+ * libhstu_hip.so so that the attention library does not depend on hipBLASLt.
  * Plain pointers and sizes; device pointers on the current HIP device; asynchronous on the stream given.
  */
 #ifndef HSTU_LINEAR_H_
@@ -43,8 +45,12 @@ typedef struct HstuUqvkArgs {
     int32_t heads, attn_dim, hidden_dim;  /* n_out = (2 * hidden_dim + 2 * attn_dim) * heads */
     int32_t dtype;             /* 0 = bf16, 1 = fp16 (HstuDtype of hstu_hip.h) */
     void* workspace;           /* hstu_uqvk_workspace_bytes() bytes, 256-byte aligned: the normalised x and the
-                                  GEMM's scratch */
+                                  GEMM's scratch (unused by the fused kernel; may then be NULL) */
     int64_t workspace_bytes;
+    int32_t path;              /* 0 = automatic: the fused kernel (layer norm, product, bias, SiLU in one pass, the
+                                  normalised rows held in registers) when d_model is 128, 256, 384 or 512 and
+                                  hidden_dim * heads and n_out are multiples of 128, else the library path;
+                                  1 = library path (layer-norm kernel + hipBLASLt); 2 = fused kernel or status -6 */
 } HstuUqvkArgs;
 
 size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* args);

@@ -148,13 +148,26 @@ def test_layer_norm_kernel(pkg, dev, L, d_model, dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("L,d_model,H,attn,hidden", [(300, 512, 4, 128, 128), (1, 64, 1, 16, 16), (1000, 128, 2, 32, 64), (257, 256, 4, 64, 32)])
-def test_compute_uqvk(pkg, dev, L, d_model, H, attn, hidden, dtype):
+@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize(
+    "L,d_model,H,attn,hidden",
+    # the first five shapes qualify for the fused kernel (d_model in 128..512 by 128, hidden * H and n_out multiples of 128)
+    [(300, 512, 4, 128, 128), (1000, 128, 2, 32, 64), (257, 256, 4, 64, 32), (1, 384, 1, 64, 128), (2049, 512, 2, 64, 64),
+     (1, 64, 1, 16, 16), (130, 512, 3, 16, 32), (77, 192, 2, 64, 64)],
+)
+def test_compute_uqvk(pkg, dev, L, d_model, H, attn, hidden, dtype, path):
     """Against the fp32 oracle, and tightly against the oracle with the reference's one intermediate rounding (the
-    normalised x in the input type)."""
-    print(f"[case] uqvk {L} {d_model} {H} {attn} {hidden} {dtype}", flush=True)
+    normalised x in the input type); `path` 0 lets the library choose (fused kernel where the shape allows), 1 forces
+    the layer-norm kernel + hipBLASLt."""
+    print(f"[case] uqvk {L} {d_model} {H} {attn} {hidden} {dtype} path={path}", flush=True)
     x, nw, nb, w, b = _inputs(L + d_model + attn, L, d_model, H, attn, hidden, dtype)
-    u, q, k, v = pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, attn, hidden, w.to(dev), b.to(dev))
+    fused_shape = d_model in (128, 256, 384, 512) and (hidden * H) % 128 == 0 and ((2 * hidden + 2 * attn) * H) % 128 == 0
+    if path == 0 and fused_shape:
+        path = 2  # the automatic choice must be the fused kernel here: asking for it explicitly may not fail
+    if path == 0 and not fused_shape:
+        with pytest.raises(NotImplementedError):
+            pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, attn, hidden, w.to(dev), b.to(dev), path=2)
+    u, q, k, v = pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, attn, hidden, w.to(dev), b.to(dev), path=path)
     torch.cuda.synchronize()
     assert u.shape == (L, hidden * H) and q.shape == (L, H, attn) and k.shape == (L, H, attn) and v.shape == (L, H, hidden)
     assert u.dtype == dtype and q.stride(2) == 1 and (L == 1 or q.stride(0) == (2 * hidden + 2 * attn) * H)
