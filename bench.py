@@ -25,7 +25,7 @@ HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced ag
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
 # counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
 MEASURED_TRAFFIC_BYTES = {"headline": 2.414e9, "cfg2": 0.827e9, "cfg3": 1.383e9, "cfg4": 0.249e9, "cfg5": 2.281e9,
-                          "kvcat": 0.173e9, "kvtail": 0.0168e9, "uqvk": 5.549e9, "layernorm": 1.074e9, "output": 5.839e9,
+                          "kvcat": 0.173e9, "kvtail": 0.0168e9, "uqvk": 2.953e9, "layernorm": 1.074e9, "output": 5.839e9,
                           "normmul": 2.684e9, "bwd": 6.250e9}
 
 
@@ -207,10 +207,11 @@ def run_linear(name, args, pkg, torch):
         nw, nb = rnd(d_model, scale=0.1, shift=1.0), rnd(d_model, scale=0.1)
         w, b = rnd(d_model, n_out, scale=1.0 / d_model**0.5), rnd(n_out, scale=0.1)
         if name == "uqvk":
-            step = lambda: hstu_compute.hstu_compute_uqvk(x, nw, nb, 1e-6, H, D, D, w, b)  # noqa: E731
+            step = lambda: hstu_compute.hstu_compute_uqvk(x, nw, nb, 1e-6, H, D, D, w, b, path=args.uqvk_path)  # noqa: E731
             cpu = lambda r: uqvk_oracle.compute_uqvk(x[:r].float().cpu(), nw.float().cpu(), nb.float().cpu(), 1e-6, H, D, D, w.float().cpu(), b.float().cpu())  # noqa: E731
             flops, nbytes = 2.0 * L * d_model * n_out, 2.0 * (L * d_model + d_model * n_out + L * n_out)
-            kernel = "hstu_layer_norm_kernel + 2 hipBLASLt GEMMs (bias, bias + SiLU epilogues)"
+            kernel = ("hstu_layer_norm_kernel + 2 hipBLASLt GEMMs (bias, bias + SiLU epilogues)" if args.uqvk_path == 1
+                      else "hstu_uqvk_fused_kernel")
             metric = "hstu_compute_uqvk fwd TFLOP/s (524288 tokens, d_model 512 -> 2048)"
         else:
             step = lambda: hstu_compute.layer_norm(x, nw, nb, 1e-6)  # noqa: E731
@@ -245,7 +246,10 @@ def run_linear(name, args, pkg, torch):
     else:
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
         value, unit = round(gbs, 1), "GB/s"
-    roof.update({"traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel, "kernel_ms": round(ev_ms, 4),
+    traffic = MEASURED_TRAFFIC_BYTES.get(name)
+    if name == "uqvk" and args.uqvk_path == 1:
+        traffic = 5.549e9  # the library path: the normalised operand written, then fetched 2-3 times
+    roof.update({"traffic": traffic, "kernel": kernel, "kernel_ms": round(ev_ms, 4),
                  "algorithmic_flops": flops, "algorithmic_bytes": nbytes, "hbm_gbs_algorithmic": round(gbs, 1)})
     line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
@@ -344,6 +348,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="headline")
     ap.add_argument("--tile-config", type=int, default=0)
+    ap.add_argument("--uqvk-path", type=int, default=0, help="workload uqvk: 0 / 2 = fused kernel, 1 = layer-norm kernel + hipBLASLt")
     ap.add_argument("--kv-splits", type=int, default=0, help="0 = the library's own rule, 1 = off, 2..8 = forced")
     ap.add_argument("--fused-buffer", action="store_true", help="q/k/v as column slices of one [L,H,3D] buffer")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

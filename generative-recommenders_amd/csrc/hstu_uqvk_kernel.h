@@ -4,18 +4,18 @@
 // (hstu_compute_uqvk of the reference, ops/hstu_compute.py:54-104; LN with fp32 statistics and its result rounded to the
 // input type, ops/pytorch/pt_layer_norm.py:24-39).
 //
-// The depth of this product (d_model, at most 512) is small enough for a wave to keep 64 normalised rows in
-// registers for the whole kernel (one wave per SIMD, 512 registers per lane): they are the B operands of every MFMA
-// (lane = row, 8 consecutive k per 16-deep step; two blocks of 32 rows, so every A operand read from LDS feeds two
-// MFMAs), loaded from HBM exactly once and normalised in place -- the normalised matrix never exists in memory.
-// W streams through LDS in tiles of 128 k x 128 n (32 KB, three slots, one barrier per tile) copied with
+// The depth of this product (d_model, at most 512) is small enough for a wave to keep its 32 normalised rows in
+// registers for the whole kernel: they are the B operand of every MFMA (lane = row, 8 consecutive k per 16-deep
+// step), loaded from HBM exactly once and normalised in place -- the normalised matrix never exists in memory.
+// W streams through LDS in tiles of 64 k x 128 n (16 KB, three slots, one barrier per tile) copied with
 // global_load_lds_dwordx4, and is read transposed (ds_read_b64_tr_b16) as the A operand:
 //     C^T[n, r] += W^T[n, k] . LN(x)^T[k, r]
 // so that a lane ends up with one output row and, per 32-column block, four runs of four consecutive columns -- the
-// accumulator layout of the attention kernels.  A workgroup of 4 waves owns 256 rows and walks all of W once:
-// for each block of 128 output columns, four k tiles of 64 MFMAs per wave, then the epilogue (bias from LDS, SiLU for
-// the u columns, rounding, a transposition through a per-wave LDS area so that every store instruction covers whole
-// 128-byte lines).  W (2 MB for 512 x 2048) stays in every XCD's L2.
+// accumulator layout of the attention kernels.  A workgroup of 4 waves owns 128 rows and walks all of W once (two
+// workgroups per CU): for each block of 128 output columns, d_model / 64 k tiles of 16 MFMAs per wave, then the
+// epilogue (bias from LDS, SiLU for the u columns, rounding, a transposition through a per-wave LDS area so that
+// every store instruction covers whole 128-byte lines).  W (2 MB for 512 x 2048) stays in every XCD's L2.
+// Stores count in the same counter as the copies (vmcnt), so the wait after an epilogue leaves room for them.
 #pragma once
 #include "hstu_common.h"
 
@@ -205,7 +205,6 @@ __global__ __launch_bounds__(kUqvkWaves * 64, 2) void hstu_uqvk_fused_kernel(con
                     }
                     *HSTU_LDS(elem4, stage + l32 * kUqvkStageRow + (d2 * 32 + r4 * 8 + g * 4) * 2) = o4;
                 }
-                __builtin_amdgcn_sched_barrier(0);  // keeps the live temporaries of the epilogue to one 32-column block
             }
             // 8 lanes cover one row's 128 bytes, 8 rows per instruction
             const int chunk = lane & 7, rsub = lane >> 3;
@@ -216,7 +215,6 @@ __global__ __launch_bounds__(kUqvkWaves * 64, 2) void hstu_uqvk_fused_kernel(con
                 if (row0 + rg * 32 + row < p.rows)
                     *(i32x4_t*)(p.out + ((row0 + rg * 32 + row) * p.n_out + c * kUqvkTileN + hf * 64) * 2 + chunk * 16) = v;
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
