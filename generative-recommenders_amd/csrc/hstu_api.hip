@@ -276,6 +276,20 @@ extern "C" __attribute__((visibility("hidden"))) void hstu_hip_set_last_error(co
     set_last_error(what, (hipError_t)hip_error);
 }
 
+// order[rank] = sequence index, longest first, for the backward entry point's schedule; 0 or HSTU_ERR_LAUNCH
+extern "C" __attribute__((visibility("hidden"))) int hstu_hip_launch_rank(const void* offsets, int offsets_i64, int batch, int* order,
+                                                                          void* stream) {
+    const unsigned blocks = (unsigned)(((long long)batch * 64 + 255) / 256);
+    hipLaunchKernelGGL(hstu::hstu_prep_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, offsets, offsets_i64, batch, order,
+                       (int*)nullptr, 0);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_last_error("rank kernel launch", e);
+        return HSTU_ERR_LAUNCH;
+    }
+    return HSTU_OK;
+}
+
 extern "C" {
 
 int hstu_hip_version(void) { return 100; }

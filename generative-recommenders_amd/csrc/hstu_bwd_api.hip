@@ -12,6 +12,8 @@
 // defined with the forward entry points (hstu_api.hip); internal to the library
 extern "C" __attribute__((visibility("hidden"))) int hstu_hip_device_is_gfx950(void);
 extern "C" __attribute__((visibility("hidden"))) void hstu_hip_set_last_error(const char* what, int hip_error);
+extern "C" __attribute__((visibility("hidden"))) int hstu_hip_launch_rank(const void* offsets, int offsets_i64, int batch, int* order,
+                                                                          void* stream);
 
 namespace {
 
@@ -128,7 +130,13 @@ extern "C" int hstu_hip_mha_bwd(const HstuFwdArgs* a, const HstuBwdGrads* g, voi
     p.pairs_per_xcd = (int)pairs_per_xcd;
     p.slots_per_xcd = (int)slots;
 
-    // `sort_by_length` is a scheduling hint only; the backward kernels take the sequences in batch order
+    // `sort_by_length`: long sequences first (their blocks are the long-running ones); needs 4 * batch bytes of workspace
+    if (a->sort_by_length && a->batch >= 2 && a->batch <= 8192 && a->workspace &&
+        (size_t)a->workspace_bytes >= (size_t)a->batch * sizeof(int)) {
+        rc = hstu_hip_launch_rank(a->seq_offsets, a->seq_offsets_i64, a->batch, (int*)a->workspace, stream_);
+        if (rc != HSTU_OK) return rc;
+        p.order = (const int*)a->workspace;
+    }
     if (a->dtype == HSTU_BF16) return launch_bwd_dim<hstu::Bf16>(bp, a->dqk, a->dv, stream);
     return launch_bwd_dim<hstu::Fp16>(bp, a->dqk, a->dv, stream);
 }

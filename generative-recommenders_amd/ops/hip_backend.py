@@ -306,8 +306,10 @@ def mha_bwd(
     max_attn_len: int,
     contextual_seq_len: int,
     min_full_attn_seq_len: int,
+    sort_by_length: bool = True,
 ) -> None:
-    """Fill ``dq``, ``dk``, ``dv`` on the current stream of ``q.device`` (full attention only)."""
+    """Fill ``dq``, ``dk``, ``dv`` on the current stream of ``q.device`` (full attention only).  ``sort_by_length``
+    starts the long sequences first; it never changes the result."""
     a = HstuFwdArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), None
     a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
@@ -327,6 +329,10 @@ def mha_bwd(
     a.max_attn_len, a.contextual_seq_len, a.min_full_attn_seq_len = max_attn_len, contextual_seq_len, min_full_attn_seq_len
     a.dtype = _dtype_code(q.dtype)
     a.q_scale = a.k_scale = a.v_scale = 1.0
+    workspace = None
+    if sort_by_length and a.batch >= 2:
+        workspace = torch.empty(4 * a.batch, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes, a.sort_by_length = workspace.data_ptr(), 4 * a.batch, 1
     g = HstuBwdGrads()
     g.dout, g.dq, g.dk, g.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     g.do_row_stride, g.do_head_stride = dout.stride(0), dout.stride(1)

@@ -144,7 +144,8 @@ const char* hstu_hip_tile_config_name(int id);
  * needed except its inputs: the scores are recomputed.  Every row of dq / dk / dv that belongs to a sequence is
  * written; no atomics, so the result is bit-identical from run to run.  The gradients have the layout rules of
  * q / k / v: 16-byte aligned base, row and head strides in elements and multiples of 8, innermost stride 1.
- * No workspace is used; `sort_by_length` (a scheduling hint) is ignored.
+ * `sort_by_length` (a scheduling hint: long sequences first) takes effect when `args->workspace` holds at least
+ * 4 * batch bytes; nothing else uses the workspace.
  */
 typedef struct HstuBwdGrads {
     const void* dout;  /* [total_q, H, dv] */

@@ -195,6 +195,41 @@ def test_backward_is_deterministic_and_takes_views(pkg, dev):
     assert torch.equal(out.detach(), b[0])
 
 
+VARIANT_CASES = [
+    # lengths, H, dqk, dv, mask kwargs
+    ([700, 300, 1, 513], 2, 128, 128, {}),
+    ([256, 255, 257, 0, 64], 2, 64, 64, {}),
+    ([1000], 1, 128, 128, dict(max_attn_len=100)),
+    ([640, 200], 2, 32, 64, dict(contextual_seq_len=150)),
+    ([900, 450], 2, 128, 128, dict(num_targets=torch.tensor([200, 449]), max_attn_len=64, contextual_seq_len=5)),
+    ([300, 300], 1, 16, 16, dict(num_targets=torch.tensor([300, 0]))),
+    ([2048 + 17], 1, 128, 128, dict(num_targets=torch.tensor([33]), max_attn_len=700, min_full_attn_seq_len=50)),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("ci", range(len(VARIANT_CASES)))
+def test_backward_through_the_backend_entry_point(pkg, dev, ci):
+    """The backend's direct entry point (no autograd), gradients pre-filled with a sentinel: every row of every sequence
+    must be overwritten."""
+    from generative_recommenders_amd.ops import hip_backend
+
+    lengths, H, dqk, dv, kw = VARIANT_CASES[ci]
+    print(f"[case] bwd direct {ci} {lengths}", flush=True)
+    q, k, v, dout, offsets = _inputs(100 + ci, lengths, H, dqk, dv, torch.bfloat16)
+    N, alpha = max(lengths) + 1, 1.0 / dqk**0.5
+    ref = G.closed_form_grads(N, alpha, q, k, v, offsets, dout, **kw)
+    qd, kd, vd, dd, od = (t.to(dev) for t in (q, k, v, dout, offsets))
+    tg = kw.get("num_targets")
+    tg = None if tg is None else tg.to(dev)
+    dq, dk, dv_ = torch.full_like(qd, 7.0), torch.full_like(kd, 7.0), torch.full_like(vd, 7.0)
+    hip_backend.mha_bwd(dd, qd, kd, vd, dq, dk, dv_, od, tg, N, alpha, kw.get("max_attn_len", 0), kw.get("contextual_seq_len", 0),
+                        kw.get("min_full_attn_seq_len", 0))
+    torch.cuda.synchronize()
+    for name, x, r in zip(("dq", "dk", "dv"), (dq, dk, dv_), ref):
+        _close(x, r, name)
+
+
 @pytest.mark.gpu
 def test_backward_of_a_long_sequence(pkg, dev):
     """4096 rows: 32 key blocks x 64 query tiles per pair, the shape the bench workload has per sequence."""
