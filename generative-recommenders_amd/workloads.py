@@ -115,7 +115,7 @@ def algorithmic_bytes(wl: Workload) -> float:
 
 
 def make_workload(name: str) -> Workload:
-    """The BASELINE configurations by name: ``cfg1`` .. ``cfg5`` and ``headline``."""
+    """The benchmark configurations by name: ``cfg1`` .. ``cfg5`` and ``headline``."""
     if name == "cfg1":
         rng = np.random.default_rng(1001)
         return Workload(name, 8, 2, 32, 32, 128, rng.integers(16, 129, size=8), dtype="fp32", seed=1001)
