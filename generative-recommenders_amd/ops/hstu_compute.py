@@ -130,6 +130,12 @@ def _dtype_code(dt: torch.dtype) -> int:
     raise RuntimeError(f"hstu_compute only supports bf16 and fp16, got {dt}")
 
 
+def _dense16(t: torch.Tensor) -> torch.Tensor:
+    """Detached, contiguous and 16-byte aligned (a slice of a larger parameter may start anywhere)."""
+    t = t.detach().contiguous()
+    return t.clone() if t.data_ptr() % 16 != 0 else t
+
+
 def _check(x: torch.Tensor, *others: torch.Tensor) -> None:
     torch._assert(x.is_cuda, "x must be CUDA tensor")
     for t in others:
@@ -149,10 +155,11 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
     if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
         x = x.contiguous()
     out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    weight, bias = _dense16(weight), _dense16(bias)
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream(x.device).cuda_stream
         rc = lib().hstu_uqvk_layer_norm(
-            x.data_ptr(), x.stride(0), weight.detach().contiguous().data_ptr(), bias.detach().contiguous().data_ptr(), eps,
+            x.data_ptr(), x.stride(0), weight.data_ptr(), bias.data_ptr(), eps,
             out.data_ptr(), out.stride(0), x.shape[0], x.shape[1], _dtype_code(x.dtype), ctypes.c_void_p(stream),
         )
     _raise_for_status(rc)
@@ -186,8 +193,8 @@ def hstu_compute_uqvk(
     uvqk = torch.empty((x.shape[0], n_out), dtype=x.dtype, device=x.device)
     a = HstuUqvkArgs()
     a.x, a.x_row_stride = x.data_ptr(), x.stride(0)
-    nw, nb = norm_weight.detach().contiguous(), norm_bias.detach().contiguous()
-    w, b = uvqk_weight.detach().contiguous(), uvqk_bias.detach().contiguous()
+    nw, nb = _dense16(norm_weight), _dense16(norm_bias)
+    w, b = _dense16(uvqk_weight), _dense16(uvqk_bias)
     a.norm_weight, a.norm_bias, a.norm_eps = nw.data_ptr(), nb.data_ptr(), norm_eps
     a.uvqk_weight, a.uvqk_bias, a.uvqk = w.data_ptr(), b.data_ptr(), uvqk.data_ptr()
     a.rows, a.d_model = x.shape[0], x.shape[1]
@@ -224,7 +231,7 @@ def _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_di
     norm_len = num_heads if group_norm else attn.shape[1]
     torch._assert(norm_weight.shape == (norm_len,) and norm_bias.shape == (norm_len,), "norm_weight / norm_bias have the wrong length")
     attn, u = _rows_ok(attn), _rows_ok(u)
-    nw, nb = norm_weight.detach().contiguous(), norm_bias.detach().contiguous()
+    nw, nb = _dense16(norm_weight), _dense16(norm_bias)
     a = HstuOutputArgs()
     a.attn, a.attn_row_stride = attn.data_ptr(), max(attn.stride(0), attn.shape[1])
     a.u, a.u_row_stride = u.data_ptr(), max(u.stride(0), u.shape[1])
@@ -292,7 +299,7 @@ def hstu_compute_output(
     a, keep, blocks = _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_dim, concat_u, concat_x,
                                    mul_u_activation_type, group_norm, False)
     torch._assert(output_weight.shape == (blocks * attn.shape[1], x.shape[1]), "output_weight must be [blocks * heads * linear_dim, d_model]")
-    xr, w = _rows_ok(x), output_weight.detach().contiguous()
+    xr, w = _rows_ok(x), _dense16(output_weight)
     out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
     a.x, a.x_row_stride = xr.data_ptr(), max(xr.stride(0), xr.shape[1])
     a.output_weight, a.out, a.d_out = w.data_ptr(), out.data_ptr(), x.shape[1]

@@ -199,6 +199,22 @@ def test_uqvk_feeds_attention_in_place(pkg, dev):
 
 
 @pytest.mark.gpu
+def test_uqvk_takes_parameters_that_are_slices_of_larger_tensors(pkg, dev):
+    """Weights that start in the middle of a larger allocation (not 16-byte aligned) and x as a column slice."""
+    L, d_model, H, attn, hidden = 200, 256, 2, 64, 64
+    x, nw, nb, w, b = _inputs(9, L, d_model, H, attn, hidden, torch.bfloat16)
+    want = pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, attn, hidden, w.to(dev), b.to(dev))
+    pad = torch.zeros(3, dtype=torch.bfloat16)
+    nw2, nb2, b2 = (torch.cat([pad, t]).to(dev)[3:] for t in (nw, nb, b))
+    x2 = torch.cat([x, x], dim=1).to(dev)[:, d_model:]
+    print("[case] uqvk sliced parameters", flush=True)
+    got = pkg.hstu_compute_uqvk(x2, nw2, nb2, 1e-6, H, attn, hidden, w.to(dev), b2)
+    torch.cuda.synchronize()
+    for g_, w_ in zip(got, want):
+        assert torch.equal(g_, w_)
+
+
+@pytest.mark.gpu
 def test_uqvk_wrapper_rejections(pkg, dev):
     x, nw, nb, w, b = [t.to(dev) for t in _inputs(5, 16, 64, 2, 8, 8, torch.bfloat16)]
     with pytest.raises(AssertionError, match="uvqk_weight must be"):
