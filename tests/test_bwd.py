@@ -242,6 +242,82 @@ def test_backward_of_a_long_sequence(pkg, dev):
 
 
 @pytest.mark.gpu
+def test_backward_at_the_size_of_the_ragged_benchmark(pkg, dev):
+    """The third benchmark configuration (64 sequences up to 8192, window 2048, contextual prefix, targets): the
+    longest and four other sequences against the closed form."""
+    from generative_recommenders_amd import workloads
+    from generative_recommenders_amd.ops import hip_backend
+
+    print("[case] bwd cfg3 full size", flush=True)
+    wl = workloads.make_workload("cfg3")
+    inp = workloads.make_inputs(wl, dev)
+    q, k, v, offs, tg = inp["q"], inp["k"], inp["v"], inp["seq_offsets"], inp["num_targets"]
+    g = torch.Generator(device=dev).manual_seed(77)
+    dout = (torch.randn(v.shape, device=dev, generator=g) * 0.1).to(v.dtype)
+    dq, dk, dv = torch.full_like(q, 7.0), torch.full_like(k, 7.0), torch.full_like(v, 7.0)
+    hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offs, tg, wl.max_seq_len, wl.alpha, wl.max_attn_len, wl.contextual_seq_len,
+                        wl.min_full_attn_seq_len)
+    torch.cuda.synchronize()
+    order = sorted(range(wl.batch), key=lambda b: -int(wl.lengths[b]))
+    picks = [order[0], order[7], order[20], order[40], order[63]]
+    ref = G.closed_form_grads(wl.max_seq_len, wl.alpha, q.cpu(), k.cpu(), v.cpu(), offs.cpu(), dout.cpu(), num_targets=tg.cpu(),
+                              max_attn_len=wl.max_attn_len, contextual_seq_len=wl.contextual_seq_len, sequences=picks)
+    oc = offs.cpu()
+    for b in picks:
+        s0, s1 = int(oc[b]), int(oc[b + 1])
+        for name, got, r in zip(("dq", "dk", "dv"), (dq, dk, dv), ref):
+            _close(got[s0:s1], r[s0:s1], f"cfg3 sequence {b} (n = {s1 - s0}) {name}")
+    assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
+
+
+@pytest.mark.gpu
+def test_backward_and_fused_producer_in_a_hip_graph(pkg, dev):
+    """hstu_compute_uqvk (fused kernel) -> hstu_mha forward -> backward kernels captured into one HIP graph: every
+    replay, with eager work and a synchronisation in between, reproduces the eager results bit for bit."""
+    from generative_recommenders_amd.ops import hip_backend, hstu_compute
+
+    print("[case] bwd + fused producer in a hip graph", flush=True)
+    H, Dh, d_model = 2, 64, 256
+    lengths = [700, 130, 1, 420]
+    offsets = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int64).to(dev)
+    L, N = sum(lengths), 700
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((L, d_model), generator=g).bfloat16().to(dev)
+    nw, nb = torch.ones(d_model).bfloat16().to(dev), torch.zeros(d_model).bfloat16().to(dev)
+    w = (torch.randn((d_model, 4 * Dh * H), generator=g) / d_model**0.5).bfloat16().to(dev)
+    bias = (0.1 * torch.randn(4 * Dh * H, generator=g)).bfloat16().to(dev)
+    dout = (0.1 * torch.randn((L, H, Dh), generator=g)).bfloat16().to(dev)
+
+    def step():
+        u, q, k, v = hstu_compute.hstu_compute_uqvk(x, nw, nb, 1e-6, H, Dh, Dh, w, bias, path=2)
+        out = pkg.hstu_mha(N, 0.125, q, k, v, offsets)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)  # views' shapes, dense storage
+        hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offsets, None, N, 0.125, 0, 0, 0, sort_by_length=False)
+        return out, dq, dk, dv
+
+    with torch.no_grad():
+        eager = step()
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            step()
+        torch.cuda.current_stream().wait_stream(stream)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            captured = step()
+        for i in range(3):
+            for t in captured:
+                t.zero_()
+            (x * 1.0).sum().item()
+            graph.replay()
+            torch.cuda.synchronize()
+            for name, a_, b_ in zip(("out", "dq", "dk", "dv"), captured, eager):
+                assert torch.equal(a_, b_), f"replay {i}: {name}"
+
+
+@pytest.mark.gpu
 def test_backward_rejections(pkg, dev):
     q, k, v, dout, offsets = _inputs(1, [40, 24], 2, 32, 32, torch.float32)
     with pytest.raises(NotImplementedError):
