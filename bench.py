@@ -287,10 +287,16 @@ def run_bwd(name, args, pkg, workloads, torch):
     g = torch.Generator(device=dev).manual_seed(wl.seed + 1)
     dout = (torch.randn(v.shape, device=dev, generator=g) * 0.1).to(v.dtype)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    # the dS scratch is the caller's and is allocated once, as a training loop would keep it
+    stored = args.bwd_form == "stored"
+    scratch = None
+    if stored:
+        need = hip_backend.mha_bwd_workspace_bytes(q.shape[0], wl.batch, wl.heads, wl.max_seq_len)
+        scratch = torch.empty(need, dtype=torch.uint8, device=dev)
 
     def step():
         hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offsets, targets, wl.max_seq_len, wl.alpha, wl.max_attn_len,
-                            wl.contextual_seq_len, wl.min_full_attn_seq_len)
+                            wl.contextual_seq_len, wl.min_full_attn_seq_len, store_ds=False, workspace=scratch)
 
     for _ in range(args.warmup):
         step()
@@ -306,11 +312,14 @@ def run_bwd(name, args, pkg, workloads, torch):
         "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": name, "batch": wl.batch, "heads": wl.heads, "dqk": wl.dqk, "dv": wl.dv, "max_seq_len": wl.max_seq_len,
                    "total_tokens": wl.total_kv, "max_attn_len": wl.max_attn_len, "contextual_seq_len": wl.contextual_seq_len,
-                   "num_targets": wl.num_targets is not None},
+                   "num_targets": wl.num_targets is not None, "form": args.bwd_form,
+                   "scratch_bytes": 0 if scratch is None else scratch.numel()},
         "pct_mfma_peak": round(100.0 * tflops / PEAK_TFLOPS[wl.dtype], 2),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_TFLOPS[wl.dtype], "unit": "TFLOP/s",
-                     "frac": round(tflops / PEAK_TFLOPS[wl.dtype], 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name),
-                     "kernel": "hstu_bwd_dkdv_kernel + hstu_bwd_dq_kernel", "kernel_ms": round(ev_ms, 4),
+                     "frac": round(tflops / PEAK_TFLOPS[wl.dtype], 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name + ("_stored" if stored else "")),
+                     "kernel": "hstu_bwd_dkdv_kernel + " + ("hstu_bwd_dq_stored_kernel" if stored else "hstu_bwd_dq_kernel"),
+                     "kernel_ms": round(ev_ms, 4),
                      "algorithmic_flops": flops, "algorithmic_bytes": nbytes},
     }
     if not args.no_cpu:
@@ -349,6 +358,8 @@ def main():
     ap.add_argument("--workload", default="headline")
     ap.add_argument("--tile-config", type=int, default=0)
     ap.add_argument("--uqvk-path", type=int, default=0, help="workload uqvk: 0 / 2 = fused kernel, 1 = layer-norm kernel + hipBLASLt")
+    ap.add_argument("--bwd-form", choices=["stored", "recompute"], default="stored",
+                    help="workloads bwd, bwd_cfg3: dS stored in scratch memory and dq streamed from it, or the scores recomputed for dq")
     ap.add_argument("--kv-splits", type=int, default=0, help="0 = the library's own rule, 1 = off, 2..8 = forced")
     ap.add_argument("--fused-buffer", action="store_true", help="q/k/v as column slices of one [L,H,3D] buffer")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

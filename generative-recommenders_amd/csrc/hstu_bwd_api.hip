@@ -18,17 +18,31 @@ extern "C" __attribute__((visibility("hidden"))) int hstu_hip_launch_rank(const 
 namespace {
 
 constexpr int kBwdWaves = 4, kBwdTile = 64, kBwdRows = kBwdWaves * 32;
+constexpr int kStoredWaves = 8, kStoredRows = kStoredWaves * 32;  // the dQ kernel that reads stored dS
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Bytes of the dS blocks: (total rows + 32 per sequence) x H x pitch32 x 64, pitch32 = 4 * ceil(max_seq_len / 128).
+size_t ds_bytes(const HstuFwdArgs* a) {
+    const size_t pitch32 = 4 * (((size_t)a->max_seq_len + 127) / 128);
+    return ((size_t)a->total_q + 32 * (size_t)a->batch) * (size_t)a->heads * pitch32 * 64;
+}
 
 template <class TT, int DQK, int DV>
 int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
     // three tile slots for the key-stationary kernel, two for the other; + 64: transposing reads of a 16-wide tile's unused half
     constexpr int smem1 = 3 * kBwdTile * (DQK + DV) * 2 + 64, smem = 2 * kBwdTile * (DQK + DV) * 2 + 64;
-    auto k1 = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
+    constexpr int smem3 = 3 * kBwdTile * DQK * 2 + kStoredWaves * 3 * 4096;
+    auto k1 = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile, false>;
+    auto k1s = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile, true>;
     auto k2 = hstu::hstu_bwd_dq_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
+    auto k3 = hstu::hstu_bwd_dq_stored_kernel<TT, DQK, kStoredWaves, kBwdTile>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1s, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, smem3);
         if (e != hipSuccess) {
             hstu_hip_set_last_error("hipFuncSetAttribute", (int)e);
             return HSTU_ERR_LAUNCH;
@@ -36,8 +50,16 @@ int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
         attr_done = true;
     }
     const unsigned grid = (unsigned)bp.f.slots_per_xcd * 8;
-    hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
-    hipLaunchKernelGGL(k2, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
+    if (bp.ds) {
+        hipLaunchKernelGGL(k1s, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
+        hstu::BwdParams b3 = bp;  // the same items in blocks of 256 query rows
+        b3.f.num_mb = (bp.f.max_seq_len + kStoredRows - 1) / kStoredRows;
+        b3.f.slots_per_xcd = bp.f.pairs_per_xcd * b3.f.num_mb;
+        hipLaunchKernelGGL(k3, dim3((unsigned)b3.f.slots_per_xcd * 8), dim3(kStoredWaves * 64), smem3, stream, b3);
+    } else {
+        hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
+        hipLaunchKernelGGL(k2, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         hstu_hip_set_last_error("backward kernel launch", (int)e);
@@ -69,6 +91,11 @@ int launch_bwd_dim(const hstu::BwdParams& bp, int dqk, int dv, hipStream_t strea
 }
 
 }  // namespace
+
+extern "C" size_t hstu_hip_mha_bwd_workspace_bytes(const HstuFwdArgs* a) {
+    if (!a || a->batch <= 0 || a->heads <= 0 || a->max_seq_len <= 0 || a->total_q <= 0) return 0;
+    return align256((size_t)a->batch * sizeof(int)) + ds_bytes(a);
+}
 
 extern "C" int hstu_hip_mha_bwd(const HstuFwdArgs* a, const HstuBwdGrads* g, void* stream_) {
     if (!a || !g) return HSTU_ERR_NULL_POINTER;
@@ -136,6 +163,12 @@ extern "C" int hstu_hip_mha_bwd(const HstuFwdArgs* a, const HstuBwdGrads* g, voi
         rc = hstu_hip_launch_rank(a->seq_offsets, a->seq_offsets_i64, a->batch, (int*)a->workspace, stream_);
         if (rc != HSTU_OK) return rc;
         p.order = (const int*)a->workspace;
+    }
+    // enough workspace for the dS blocks: the key-stationary kernel stores them and dQ is formed from them
+    if (a->workspace && (size_t)a->workspace_bytes >= hstu_hip_mha_bwd_workspace_bytes(a) &&
+        (reinterpret_cast<uintptr_t>(a->workspace) & 255) == 0) {
+        bp.ds = (char*)a->workspace + align256((size_t)a->batch * sizeof(int));
+        bp.ds_pitch32 = 4 * ((a->max_seq_len + 127) / 128);
     }
     if (a->dtype == HSTU_BF16) return launch_bwd_dim<hstu::Bf16>(bp, a->dqk, a->dv, stream);
     return launch_bwd_dim<hstu::Fp16>(bp, a->dqk, a->dv, stream);

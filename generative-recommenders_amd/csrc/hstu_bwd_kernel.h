@@ -39,7 +39,75 @@ struct BwdParams {
     int64_t do_rs, do_hs, dq_rs, dq_hs, dk_rs, dk_hs, dv_rs, dv_hs;  // strides in elements
     float pscale;  // dV = pscale * sum(p dOut), p = t * sigma with t = c1 * s:  (alpha / N) / c1
     float gscale;  // dQ, dK = gscale * sum(...):  alpha / N
+    // Stored-dS mode (both null / 0 otherwise): the key-stationary kernel writes every block of dS it forms, rounded
+    // to the operand type, and hstu_bwd_dq_stored_kernel reads them back instead of forming S and dP again.
+    char* ds;
+    int ds_pitch32;  // blocks of 32 keys per row of blocks: 4 * ceil(max_seq_len / 128)
 };
+
+// Where the dS blocks of one (sequence, head) pair live.  A block is 32 query rows x 32 keys, 2 KB, in the register
+// image of the wave that formed it: half h (query rows 16 h ..), lane (key c = lane % 32, g = lane / 32) holds 16 bytes
+// = query rows 16 h + 8 j + 4 g + {0..3}, j = 0, 1, at 16-byte position 64 h + ((2 c + g) ^ 8 h) -- every store covers
+// a contiguous KB, and the XOR makes the transposing LDS reads of the consumer conflict-free.  Sequence b owns the
+// bytes of (len_b + 32) rows x H x pitch32 x 64, enough for H x ceil(len_b / 32) x pitch32 blocks, starting at
+// (offset_b + 32 b) rows; block (h, qb, kb) is number (h * nqb + qb) * pitch32 + kb of them.
+__device__ __forceinline__ char* ds_pair_base(const BwdParams& bp, const Work& W, int n) {
+    const int64_t row_units = (W.seq_start + 32 * (int64_t)W.b) * bp.f.H * bp.ds_pitch32;
+    const int nqb = (n + 31) >> 5;
+    return bp.ds + row_units * 64 + (int64_t)W.h * nqb * bp.ds_pitch32 * 2048;
+}
+
+constexpr int kKeyBlock = 128, kQueryTile = 64;  // geometry of the key-stationary kernel
+
+// The tiles of 64 query rows that the key-stationary kernel visits for the 128 keys starting at S0: rows at or after
+// the first key (all rows if a contextual prefix sees every key), up to the last row whose window still reaches the
+// block (targets sit at id max_id); inside that range a tile without a valid pair is passed over.
+struct KeyBlockWalk {
+    int first, end;
+    bool scan;
+    __device__ __forceinline__ void init(const SeqMask& M, bool has_targets, int S0, int n) {
+        const int S1 = (S0 + kKeyBlock < n ? S0 + kKeyBlock : n) - 1;
+        int q_hi = n - 1;
+        if (M.w > 0 && M.f == 0) {
+            const int id1 = M.id(S1);
+            const bool targets_reach = has_targets && M.max_id - id1 <= M.w;
+            if (!targets_reach) {
+                const int hi = id1 + M.w + M.shift;
+                q_hi = hi < q_hi ? hi : q_hi;
+            }
+        }
+        end = q_hi / kQueryTile + 1;
+        first = M.c > 0 ? 0 : S0 / kQueryTile;
+        scan = M.w > 0 || M.c > 0 || has_targets;
+    }
+    __device__ __forceinline__ bool visits(const SeqMask& M, int jt, int S0, int n) const {
+        if (jt < first || jt >= end) return false;
+        if (!scan) return true;
+        const int r1 = (jt + 1) * kQueryTile < n ? (jt + 1) * kQueryTile - 1 : n - 1;
+        return M.classify(jt * kQueryTile, r1, S0, kKeyBlock) != 0;
+    }
+    __device__ __forceinline__ int next(const SeqMask& M, int jt, int S0, int n) const {
+        jt = jt < first ? first : jt;
+        while (jt < end && !visits(M, jt, S0, n)) ++jt;
+        return jt < end ? jt : end;
+    }
+};
+
+// Class of the block of 32 query rows from r0 against the 32 keys from s0 (both inside the sequence or past its end):
+// 0 nothing valid, 1 masked, 2 all valid.  The key-stationary kernel stores dS for a block iff the class is not 0 and
+// its walk visits the tile of the block.  `plain` (causal only: no window, contextual prefix or targets) takes a
+// shortcut with the same answers.
+__device__ __forceinline__ int block_class32(const SeqMask& M, bool plain, int r0, int s0, int n) {
+    if (r0 >= n || s0 >= n) return 0;
+    if (plain) {
+        if (r0 + 31 < s0) return 0;
+        return (r0 > s0 + 31 && r0 + 31 < n && s0 + 31 < n) ? 2 : 1;
+    }
+    const int r1 = r0 + 31 < n ? r0 + 31 : n - 1;
+    int cls = M.classify(r0, r1, s0, 32);
+    if (cls == 2 && r0 + 31 >= n) cls = 1;
+    return cls;
+}
 
 // Chunk swizzle for a tile read both ways: the bits the transposing read needs (swz_v) plus row bit 3 in chunk bit 0,
 // which makes the 16 rows of a ds_read_b128 land in 16 different 16-byte slots and changes nothing for a transposing
@@ -177,26 +245,24 @@ struct TwoChains {
     static constexpr int index(int k) { return k < 2 * M ? k / 2 : k - M; }
 };
 
-// The key-stationary kernel has two 128-row accumulators and K, V in registers: one wave per SIMD.  A wave alone
-// must therefore overlap its own matrix and VALU work, which it does by software pipelining over blocks of 32
-// query rows: phase A issues the S and dP products of the NEXT block, one MFMA at a time, each followed by the
-// pointwise work (sigmoid, slope, mask, rounding) on one accumulator element of the CURRENT block; phase B then
-// issues the dV and dK products of the current block.  LDS operands are requested PD MFMAs ahead.  Tiles of 64
-// query rows sit in three LDS slots; the one barrier per tile comes after the first block of a tile has gone through
-// phase B, when nobody can still read the tile before it, whose slot the next copy overwrites.
-// Blocks are skipped per wave only in whole phases (a block with no valid pair for the wave's keys gets neither
-// products nor pointwise work); the barrier count per tile is the same for every wave.
-template <class TT, int DQK, int DV, int NW, int BN>
+// The key-stationary kernel has two 128-row accumulators and K, V in registers: one wave per SIMD, and on this
+// hardware a wave's own VALU work does not run while its MFMAs do, so what counts is the length of the one instruction
+// stream.  It is software-pipelined over blocks of 32 query rows with three blocks in flight: every step issues the
+// S and dP products of block i + 1, the pointwise work (sigmoid, slope, rounding) on block i, and the dV and dK
+// products of block i - 1, slot by slot (two MFMAs, their LDS operand requests, one accumulator element), with the
+// copies of the tile after next spread over the slots.  Tiles of 64 query rows sit in three LDS slots; the one barrier
+// per tile comes when nobody can still read the tile before, whose slot the next copy overwrites.
+template <class TT, int DQK, int DV, int NW, int BN, bool STORE>
 __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdParams bp) {
     typedef typename TT::vec8 vec8;
-    static_assert(BN == 64, "two blocks of 32 query rows per tile");
+    static_assert(BN == kQueryTile && NW * 32 == kKeyBlock, "two blocks of 32 query rows per tile, four waves of 32 keys");
     const FwdParams& p = bp.f;
     constexpr int BM = NW * 32;  // key rows per workgroup
     constexpr int KS = DQK / 16, VS = DV / 16, DTK = (DQK + 31) / 32, DTV = (DV + 31) / 32;
     constexpr int QROW = DQK * 2, OROW = DV * 2;
     constexpr int QTILE = BN * QROW, OTILE = BN * OROW, STAGE = QTILE + OTILE;
     constexpr int NT = NW * 64;
-    constexpr int PD = 3;  // LDS operands in flight ahead of the MFMA that uses them
+    constexpr int PD = 2;  // LDS operands in flight ahead of the MFMA that uses them
     typedef TwoChains<KS, VS> OpsA;
     typedef TwoChains<2 * DTV, 2 * DTK> OpsB;
     extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -209,40 +275,49 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
     if (!bwd_decode<BM>(p, W, blockIdx.x, true)) return;
     const SeqMask& M = W.M;
     const int n = W.n;
-    const int S0 = W.R0, S1 = W.R1;  // key rows of the workgroup (inclusive)
-    const int wS0 = S0 + wave * 32;  // first key row of the wave; the wave has no keys if wS0 > S1
+    const int S0 = W.R0;             // first key row of the workgroup
+    const int wS0 = S0 + wave * 32;  // first key row of the wave; the wave has no keys if wS0 >= n
 
-    // query tiles [.., jt_end): rows at or after the first key (all rows if a contextual prefix sees every key), up
-    // to the last row whose window still reaches the block (targets sit at id max_id)
-    int q_hi = n - 1;
-    if (M.w > 0 && M.f == 0) {
-        const int id1 = M.id(S1);
-        const bool targets_reach = p.targets != nullptr && M.max_id - id1 <= M.w;
-        if (!targets_reach) {
-            const int hi = id1 + M.w + M.shift;
-            q_hi = hi < q_hi ? hi : q_hi;
-        }
-    }
-    const int jt_end = q_hi / BN + 1;
-    auto next_tile = [&](int jt) {
-        if (W.skip_scan)
-            while (jt < jt_end) {
-                const int r1 = (jt + 1) * BN < n ? (jt + 1) * BN - 1 : n - 1;
-                if (M.classify(jt * BN, r1, S0, BM) != 0) break;
-                ++jt;
-            }
-        return jt;
-    };
+    KeyBlockWalk walk;
+    walk.init(M, p.targets != nullptr, S0, n);
+    const int jt_end = walk.end;
+    auto next_tile = [&](int jt) { return walk.next(M, jt, S0, n); };
 
     const char* qbase = p.q + (W.seq_start * p.q_rs + (int64_t)W.h * p.q_hs) * 2;
     const char* obase = bp.dout + (W.seq_start * bp.do_rs + (int64_t)W.h * bp.do_hs) * 2;
     const int64_t q_rsb = p.q_rs * 2, o_rsb = bp.do_rs * 2;
+    // per-lane byte offsets of this wave's copies inside a tile that lies wholly inside the sequence (32 bits: usable
+    // when 64 rows stay below 2 GB, else every tile takes the general path)
+    const bool fast_copy = q_rsb < (1 << 24) && o_rsb < (1 << 24);
+    constexpr int QCP = (BN * (QROW / 16) / 64 + NW - 1) / NW, OCP = (BN * (OROW / 16) / 64 + NW - 1) / NW;
+    unsigned qoff[QCP], ooff[OCP];
+#pragma unroll
+    for (int i = 0; i < QCP; ++i) {
+        const int pos = (wave + i * NW) * 64 + lane, row = pos / (QROW / 16);
+        qoff[i] = (unsigned)(row * (int)q_rsb + (((pos % (QROW / 16)) ^ swz_u<QROW / 16>(row)) * 16));
+    }
+#pragma unroll
+    for (int i = 0; i < OCP; ++i) {
+        const int pos = (wave + i * NW) * 64 + lane, row = pos / (OROW / 16);
+        ooff[i] = (unsigned)(row * (int)o_rsb + (((pos % (OROW / 16)) ^ swz_u<OROW / 16>(row)) * 16));
+    }
     auto copy_tile = [&](int jt, int slot) {
+        if (fast_copy && (jt + 1) * BN <= n) {
+            const char* qb = qbase + (int64_t)jt * BN * q_rsb;
+            const char* ob = obase + (int64_t)jt * BN * o_rsb;
+#pragma unroll
+            for (int i = 0; i < QCP; ++i)
+                if (wave + i * NW < BN * (QROW / 16) / 64) global_load_lds16_soff(qb, qoff[i], smem + slot * STAGE + (wave + i * NW) * 1024);
+#pragma unroll
+            for (int i = 0; i < OCP; ++i)
+                if (wave + i * NW < BN * (OROW / 16) / 64) global_load_lds16_soff(ob, ooff[i], smem + slot * STAGE + QTILE + (wave + i * NW) * 1024);
+            return;
+        }
         load_tile_u<BN, QROW, NT>(qbase, q_rsb, jt * BN, n - 1, smem + slot * STAGE, wave, lane);
         load_tile_u<BN, OROW, NT>(obase, o_rsb, jt * BN, n - 1, smem + slot * STAGE + QTILE, wave, lane);
     };
 
-    int t_cur = next_tile(M.c > 0 ? 0 : S0 / BN);
+    int t_cur = next_tile(0);
     int t_nxt = t_cur < jt_end ? next_tile(t_cur + 1) : jt_end;
     if (t_cur < jt_end) copy_tile(t_cur, 0);
     if (t_nxt < jt_end) copy_tile(t_nxt, 1);
@@ -267,110 +342,127 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
     }
 
     // class of the block of 32 query rows starting at r0 against this wave's keys: 0 nothing valid, 1 masked, 2 all valid
-    auto block_class = [&](int r0) {
-        if (r0 >= n || wS0 > S1) return 0;
-        const int r1 = r0 + 31 < n ? r0 + 31 : n - 1;
-        int cls = M.classify(r0, r1, wS0, 32);
-        if (cls == 2 && r0 + 31 >= n) cls = 1;
-        return cls;
-    };
+    auto block_class = [&](int r0) { return block_class32(M, !walk.scan, r0, wS0, n); };
 
-    // Phase A.  MFMA: issue S and dP of the block whose Q / dOut rows start at qn / on into (s_n, dp_n).
-    // PW (0 none, 1 masked, 2 all valid): P and dS of the block held in (s_c, dp_c), whose first query row is r0_c,
-    // packed into pb / dsb.
-    auto phase_a = [&](auto mfma_c, auto pw_c, const char* qn, const char* on, f32x16_t& s_n, f32x16_t& dp_n, const f32x16_t& s_c,
-                       const f32x16_t& dp_c, int r0_c, vec8 (&pb)[2], vec8 (&dsb)[2]) __attribute__((always_inline)) {
-        constexpr bool MFMA = decltype(mfma_c)::value;
-        constexpr int PW = decltype(pw_c)::value;
-        constexpr int NA = OpsA::N;
-        auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
+    // stored-dS mode: this lane's slot in the blocks of the wave's 32 keys (block row 0 of the pair)
+    char* dsw = nullptr;
+    if constexpr (STORE) dsw = ds_pair_base(bp, W, n) + (int64_t)(wS0 >> 5) * 2048 + (2 * l32 + g) * 16;
+    const int64_t ds_qb_stride = (int64_t)bp.ds_pitch32 * 2048;
+
+    // One step of the pipeline, in 16 slots (one per accumulator element of a block).  Three blocks of 32 query rows are
+    // in flight: A -- the S and dP products of the block whose Q / dOut rows start at qn / on, into (s_n, dp_n);
+    // PW -- P and dS of the block held in (s_c, dp_c), packed into (pb_o, dsb_o) WITHOUT the mask; B -- dV^T += dOut^T P
+    // and dK^T += Q^T dS of the block before, whose rows start at qb / ob and whose packed P, dS are (pb_i, dsb_i).
+    // The matrix pipe runs A and B while the VALU does PW; LDS operands are requested PD MFMAs ahead in each stream.
+    // There is one instruction stream for all kinds of blocks (variants chosen at run time would meet again with the
+    // accumulators in different registers, and the copies cost more than the work saved): a block without a valid pair
+    // for the wave's keys, or past the end of the sequence, runs on whatever rows are there, and `apply_mask` below then
+    // clears what must not count.
+    auto step = [&](const char* qn, const char* on, f32x16_t& s_n, f32x16_t& dp_n, const f32x16_t& s_c, const f32x16_t& dp_c,
+                    vec8 (&pb_o)[2], vec8 (&dsb_o)[2], const char* qb, const char* ob, const vec8 (&pb_i)[2], const vec8 (&dsb_i)[2],
+                    int r0_b, bool store_b, bool do_copy, const char* cq, const char* co, char* cl) __attribute__((always_inline)) {
+        constexpr int NA = OpsA::N, NB = OpsB::N, NCP = QCP + OCP;
+        auto load_a = [&](int k) __attribute__((always_inline)) -> vec8 {
             return OpsA::first(k) ? *HSTU_LDS(const vec8, qn + qrow[OpsA::index(k)]) : *HSTU_LDS(const vec8, on + orow[OpsA::index(k)]);
         };
-        vec8 fr[PD];
-        if constexpr (MFMA) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s_n[r] = dp_n[r] = 0.f;
-#pragma unroll
-            for (int k = 0; k < PD && k < NA; ++k) fr[k] = load_op(k);
-        }
-        float pv[16], dsv[16];
-#pragma unroll
-        for (int k = 0; k < NA; ++k) {
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (MFMA) {
-                if (OpsA::first(k)) s_n = TT::mfma(fr[k % PD], kreg[OpsA::index(k)], s_n);
-                else dp_n = TT::mfma(fr[k % PD], vreg[OpsA::index(k)], dp_n);
-                if (k + PD < NA) fr[k % PD] = load_op(k + PD);
+        auto load_b = [&](int k) __attribute__((always_inline)) -> vec8 {
+            const int i = OpsB::index(k);
+            if (OpsB::first(k)) {
+                const char* b = ob + (i / DTV) * 16 * OROW;
+                return read_vt_operand<TT>(b + otr[0][i % DTV], b + otr[1][i % DTV]);
             }
-            if constexpr (PW != 0) {
+            const char* b = qb + (i / DTK) * 16 * QROW;
+            return read_vt_operand<TT>(b + qtr[0][i % DTK], b + qtr[1][i % DTK]);
+        };
+        vec8 fa[PD], fb[PD];
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    if (e * NA / 16 != k) continue;
-                    float pr, gr;
-                    silu_and_slope(s_c[e], pr, gr);
-                    float dsr = dp_c[e] * gr;
-                    if constexpr (PW == 1) {
-                        const bool ok = key.valid(M, r0_c + 8 * (e >> 2) + 4 * g + (e & 3));
-                        pr = ok ? pr : 0.f;
-                        dsr = ok ? dsr : 0.f;
-                    }
-                    pv[e] = pr;
-                    dsv[e] = dsr;
-                    if (e == 7 || e == 15) {
-                        float p8[8], d8[8];
+        for (int r = 0; r < 16; ++r) s_n[r] = dp_n[r] = 0.f;
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            p8[j] = pv[e - 7 + j];
-                            d8[j] = dsv[e - 7 + j];
-                        }
-                        pb[e >> 3] = TT::pack8(p8);
-                        dsb[e >> 3] = TT::pack8(d8);
+        for (int k = 0; k < PD && k < NA; ++k) fa[k] = load_a(k);
+#pragma unroll
+        for (int k = 0; k < PD && k < NB; ++k) fb[k] = load_b(k);
+        float pv[16], dsv[16];
+        auto mat = [&](int e) __attribute__((always_inline)) {
+#pragma unroll
+            for (int k = 0; k < NA; ++k) {
+                if (k * 16 / NA != e) continue;
+                if (OpsA::first(k)) s_n = TT::mfma(fa[k % PD], kreg[OpsA::index(k)], s_n);
+                else dp_n = TT::mfma(fa[k % PD], vreg[OpsA::index(k)], dp_n);
+                if (k + PD < NA) fa[k % PD] = load_a(k + PD);
+            }
+#pragma unroll
+            for (int k = 0; k < NB; ++k) {
+                if (k * 16 / NB != e) continue;
+                const int i = OpsB::index(k);
+                if (OpsB::first(k)) dvacc[i % DTV][0] = TT::mfma(fb[k % PD], pb_i[i / DTV], dvacc[i % DTV][0]);
+                else dkacc[i % DTK][0] = TT::mfma(fb[k % PD], dsb_i[i / DTK], dkacc[i % DTK][0]);
+                if (k + PD < NB) fb[k % PD] = load_b(k + PD);
+            }
+            // the copies of a tile that lies wholly inside the sequence go out one at a time between the products
+#pragma unroll
+            for (int c = 0; c < NCP; ++c) {
+                if (c * 16 / NCP != e) continue;
+                if (do_copy) {
+                    if (c < QCP) {
+                        if (wave + c * NW < BN * (QROW / 16) / 64) global_load_lds16_soff(cq, qoff[c], cl + (wave + c * NW) * 1024);
+                    } else {
+                        if (wave + (c - QCP) * NW < BN * (OROW / 16) / 64)
+                            global_load_lds16_soff(co, ooff[c - QCP], cl + QTILE + (wave + (c - QCP) * NW) * 1024);
                     }
                 }
             }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // Phase B: dV^T += dOut^T P and dK^T += Q^T dS for the block whose rows start at qc / oc.
-    auto phase_b = [&](const char* qc, const char* oc, const vec8 (&pb)[2], const vec8 (&dsb)[2]) __attribute__((always_inline)) {
-        constexpr int NB = OpsB::N;
-        auto load_op = [&](int k) __attribute__((always_inline)) -> vec8 {
-            const int i = OpsB::index(k);
-            if (OpsB::first(k)) {
-                const char* b = oc + (i / DTV) * 16 * OROW;
-                return read_vt_operand<TT>(b + otr[0][i % DTV], b + otr[1][i % DTV]);
+            if constexpr (STORE) if (store_b) {
+                char* dst = dsw + (r0_b >> 5) * ds_qb_stride;
+                if (e == 0) *(vec8*)dst = dsb_i[0];
+                if (e == 2) *(vec8*)(dst + 1024 + (((2 * l32 + g) * 16) ^ 128) - (2 * l32 + g) * 16) = dsb_i[1];
             }
-            const char* b = qc + (i / DTK) * 16 * QROW;
-            return read_vt_operand<TT>(b + qtr[0][i % DTK], b + qtr[1][i % DTK]);
         };
-        vec8 fr[PD];
+        auto pw = [&](int e) __attribute__((always_inline)) {
+            float pr, gr;
+            silu_and_slope(s_c[e], pr, gr);
+            pv[e] = pr;
+            dsv[e] = dp_c[e] * gr;
+            if (e == 7 || e == 15) {
+                float p8[8], d8[8];
 #pragma unroll
-        for (int k = 0; k < PD && k < NB; ++k) fr[k] = load_op(k);
+                for (int j = 0; j < 8; ++j) {
+                    p8[j] = pv[e - 7 + j];
+                    d8[j] = dsv[e - 7 + j];
+                }
+                pb_o[e >> 3] = TT::pack8(p8);
+                dsb_o[e >> 3] = TT::pack8(d8);
+            }
+        };
 #pragma unroll
-        for (int k = 0; k < NB; ++k) {
+        for (int e = 0; e < 16; ++e) {
             __builtin_amdgcn_sched_barrier(0);
-            const int i = OpsB::index(k);
-            if (OpsB::first(k)) dvacc[i % DTV][0] = TT::mfma(fr[k % PD], pb[i / DTV], dvacc[i % DTV][0]);
-            else dkacc[i % DTK][0] = TT::mfma(fr[k % PD], dsb[i / DTK], dkacc[i % DTK][0]);
-            if (k + PD < NB) fr[k % PD] = load_op(k + PD);
+            mat(e);
+            pw(e);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
-    typedef std::integral_constant<bool, true> Yes;
-    typedef std::integral_constant<bool, false> No;
-    typedef std::integral_constant<int, 0> Pw0;
-    typedef std::integral_constant<int, 1> Pw1;
-    typedef std::integral_constant<int, 2> Pw2;
-    // phase A with the two choices made at run time (both are wave-uniform)
-    auto run_a = [&](bool mfma, int pw, const char* qn, const char* on, f32x16_t& s_n, f32x16_t& dp_n, const f32x16_t& s_c,
-                     const f32x16_t& dp_c, int r0_c, vec8 (&pb)[2], vec8 (&dsb)[2]) __attribute__((always_inline)) {
-        if (mfma) {
-            if (pw == 2) phase_a(Yes{}, Pw2{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
-            else if (pw == 1) phase_a(Yes{}, Pw1{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
-            else phase_a(Yes{}, Pw0{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
-        } else {
-            if (pw == 2) phase_a(No{}, Pw2{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
-            else if (pw == 1) phase_a(No{}, Pw1{}, qn, on, s_n, dp_n, s_c, dp_c, r0_c, pb, dsb);
+    // Clear the entries of a packed block (first query row r0) that the mask removes: everything for class 0, the
+    // pairs the predicate rejects for class 1.  Works on the rounded values, so whatever the pointwise step made of
+    // rows that do not exist (even a NaN) goes away.
+    typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+    auto apply_mask = [&](int cls, int r0, vec8 (&pb_o)[2], vec8 (&dsb_o)[2]) __attribute__((always_inline)) {
+        if (cls == 2) return;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            u32x4_t m;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                unsigned bits = 0;
+                if (cls == 1) {
+                    const int e = 8 * h + 2 * w;
+                    const bool lo = key.valid(M, r0 + 8 * (e >> 2) + 4 * g + (e & 3));
+                    const bool hi = key.valid(M, r0 + 8 * ((e + 1) >> 2) + 4 * g + ((e + 1) & 3));
+                    bits = (lo ? 0xFFFFu : 0u) | (hi ? 0xFFFF0000u : 0u);
+                }
+                m[w] = bits;
+            }
+            pb_o[h] = __builtin_bit_cast(vec8, __builtin_bit_cast(u32x4_t, pb_o[h]) & m);
+            dsb_o[h] = __builtin_bit_cast(vec8, __builtin_bit_cast(u32x4_t, dsb_o[h]) & m);
         }
     };
 
@@ -378,41 +470,71 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first tiles have landed
         __syncthreads();
         f32x16_t sx, dpx, sy, dpy;  // block 0 of a tile lives in x, block 1 in y
-        vec8 pb[2], dsb[2];
+        vec8 pbx[2], dsbx[2], pby[2], dsby[2];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sy[r] = dpy[r] = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) pby[0][j] = pby[1][j] = dsby[0][j] = dsby[1][j] = 0;
         int slot = 0;
         int clsx = block_class(t_cur * BN);
-        run_a(clsx != 0, 0, smem, smem + QTILE, sx, dpx, sx, dpx, 0, pb, dsb);
+        // products of the first block; the other two stages run on zeros
+        step(smem, smem + QTILE, sx, dpx, sy, dpy, pbx, dsbx, smem, smem + QTILE, pby, dsby, 0, false, false, nullptr, nullptr, nullptr);
+        // Stores count in vmcnt like the tile copies, in order: the wait for a copy may leave the stores issued after
+        // it outstanding (two per block whose dV / dK products ran since).
+        int stores_x = 0;
+        int clsy_prev = 0, r0_prev = 0;
+        const char* qt_prev = smem;
         while (true) {
             const char* qt = smem + slot * STAGE;
             const char* ot = qt + QTILE;
-            // block 1 of this tile enters phase A while block 0 gets its pointwise work
+            // block 1 of this tile: products; block 0: pointwise work; block 1 of the tile before: dV, dK
             const int clsy = block_class(t_cur * BN + 32);
-            run_a(clsy != 0, clsx, qt + 32 * QROW, ot + 32 * OROW, sy, dpy, sx, dpx, t_cur * BN, pb, dsb);
-            if (clsx != 0) phase_b(qt, ot, pb, dsb);
+            step(qt + 32 * QROW, ot + 32 * OROW, sy, dpy, sx, dpx, pbx, dsbx, qt_prev + 32 * QROW, qt_prev + QTILE + 32 * OROW, pby, dsby,
+                 r0_prev, clsy_prev != 0, false, nullptr, nullptr, nullptr);
+            apply_mask(clsx, t_cur * BN, pbx, dsbx);
             const bool more = t_nxt < jt_end;
-            int t_nn = jt_end;
+            int t_nn = jt_end, cslot = 0;
+            bool inline_copy = false;
+            const char* qn = qt;  // after the last tile the products of the "next" block run on this one and are dropped
             if (more) {
-                __builtin_amdgcn_s_waitcnt(0x0F70);  // the next tile, copied during the last one, has landed
-                __syncthreads();                      // ... for every wave; and nobody reads the tile before this one any more
+                // the next tile, copied during the last one, has landed
+                const int younger = STORE ? stores_x + (clsy_prev != 0 ? 2 : 0) : 0;
+                if (younger == 4) __builtin_amdgcn_s_waitcnt(0x0F74);
+                else if (younger == 2) __builtin_amdgcn_s_waitcnt(0x0F72);
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+                __syncthreads();  // ... for every wave; and nobody reads the tile before this one any more
                 t_nn = next_tile(t_nxt + 1);
                 const int nslot = slot == 2 ? 0 : slot + 1;
-                if (t_nn < jt_end) copy_tile(t_nn, nslot == 2 ? 0 : nslot + 1);
-                clsx = block_class(t_nxt * BN);
-                const char* qn = smem + nslot * STAGE;
-                run_a(clsx != 0, clsy, qn, qn + QTILE, sx, dpx, sy, dpy, t_cur * BN + 32, pb, dsb);
-            } else {
-                run_a(false, clsy, qt, ot, sx, dpx, sy, dpy, t_cur * BN + 32, pb, dsb);
+                cslot = nslot == 2 ? 0 : nslot + 1;
+                inline_copy = fast_copy && t_nn < jt_end && (t_nn + 1) * BN <= n;
+                // a tile that reaches past the end of the sequence (the last one) is copied here, with its rows clamped
+                if (t_nn < jt_end && !inline_copy) copy_tile(t_nn, cslot);
+                // stores issued after the last copy and before the next wait for it
+                stores_x = inline_copy ? 0 : (clsx != 0 ? 2 : 0);
+                qn = smem + nslot * STAGE;
             }
-            if (clsy != 0) phase_b(qt + 32 * QROW, ot + 32 * OROW, pb, dsb);
+            // block 0 of the next tile: products; block 1 of this tile: pointwise work; block 0 of this tile: dV, dK
+            step(qn, qn + QTILE, sx, dpx, sy, dpy, pby, dsby, qt, ot, pbx, dsbx, t_cur * BN, clsx != 0, inline_copy,
+                 qbase + (int64_t)t_nn * BN * q_rsb, obase + (int64_t)t_nn * BN * o_rsb, smem + cslot * STAGE);
+            apply_mask(clsy, t_cur * BN + 32, pby, dsby);
+            clsy_prev = clsy;
+            r0_prev = t_cur * BN + 32;
+            qt_prev = qt;
             if (!more) break;
+            clsx = block_class(t_nxt * BN);
             t_cur = t_nxt;
             t_nxt = t_nn;
             slot = slot == 2 ? 0 : slot + 1;
         }
+        // dV, dK of the very last block (the other two stages run on what is there and are dropped)
+        step(qt_prev, qt_prev + QTILE, sy, dpy, sx, dpx, pbx, dsbx, qt_prev + 32 * QROW, qt_prev + QTILE + 32 * OROW, pby, dsby,
+             r0_prev, clsy_prev != 0, false, nullptr, nullptr, nullptr);
     }
     store_output<TT, DTK>(dkacc, 0, bp.dk, W.seq_start, wS0 + l32, n, bp.dk_rs, bp.dk_hs, W.h, g, bp.gscale, DQK);
     store_output<TT, DTV>(dvacc, 0, bp.dv, W.seq_start, wS0 + l32, n, bp.dv_rs, bp.dv_hs, W.h, g, bp.pscale, DV);
 }
+
+
 
 // ---- query-stationary kernel: dQ -----------------------------------------------------------------------------------
 
@@ -521,5 +643,130 @@ __global__ __launch_bounds__(NW * 64, 2) void hstu_bwd_dq_kernel(const BwdParams
     }
     store_output<TT, DTK>(dqacc, 0, bp.dq, W.seq_start, wq0 + l32, n, bp.dq_rs, bp.dq_hs, W.h, g, bp.gscale, DQK);
 }
+
+// ---- dQ from stored dS --------------------------------------------------------------------------------------------
+
+// dQ^T[d, q] += K^T dS^T with dS read back from the blocks the key-stationary kernel stored: one product instead of
+// three and no pointwise work; the kernel streams 2 bytes per (query, key) pair from HBM and is bound by that.
+// A workgroup owns NW * 32 query rows and walks the key tiles as the forward kernel does.  K tiles are shared through
+// LDS (three slots, one barrier per tile); each wave copies the two blocks of ITS 32 rows per tile straight into a
+// private LDS ring (three slots as well, so two tiles -- 2 x NW x 4 KB -- are in flight per workgroup) and reads them
+// with transposing reads: the stored image has the key in the lane and four consecutive query rows per 8 bytes, the
+// B operand wants the query row in the lane and consecutive keys.  A block is used iff the key-stationary kernel
+// stored it (same walk, same classification).
+template <class TT, int DQK, int NW, int BN>
+__global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dq_stored_kernel(const BwdParams bp) {
+    typedef typename TT::vec8 vec8;
+    static_assert(BN == 64 && TT::ES == 2, "two blocks of 32 keys per tile, 16-bit operands");
+    const FwdParams& p = bp.f;
+    constexpr int BM = NW * 32;
+    constexpr int DTK = (DQK + 31) / 32;
+    constexpr int KROW = DQK * 2, KTILE = BN * KROW, KCH = KROW / 16;
+    constexpr int KINSTR = BN * KCH / 64, KPW = (KINSTR + NW - 1) / NW;  // K copies per tile, per wave
+    constexpr int NSLOT = 3, DSBYTES = 4096;                            // per wave and slot: two blocks
+    constexpr int PER_STEP = KPW + 4;
+    static_assert(PER_STEP <= 15, "wait immediates below");
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    char* const ds_lds = smem + NSLOT * KTILE;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 5, l32 = lane & 31;
+
+    Work W;
+    if (!bwd_decode<BM>(p, W, blockIdx.x, false)) return;
+    const SeqMask& M = W.M;
+    const int n = W.n;
+    kv_tile_range(M, W.u, W.R0, W.R1, BN, W.jt_begin, W.jt_end);
+    const int jt_end = W.jt_end;
+    const int wq0 = W.m0 + wave * 32;  // the wave has no rows if wq0 >= n
+
+    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * 2;
+    const int64_t k_rsb = p.k_rs * 2;
+    // the wave's row of blocks; a wave without rows copies the last row of blocks and uses nothing of it
+    const int nqb = (n + 31) >> 5;
+    const int qb = (wq0 >> 5) < nqb ? (wq0 >> 5) : nqb - 1;
+    const char* dsrow = ds_pair_base(bp, W, n) + (int64_t)qb * bp.ds_pitch32 * 2048;
+    char* const my_ds = ds_lds + wave * (NSLOT * DSBYTES);
+
+    auto copy_step = [&](int jt, int slot) {
+        // every wave issues KPW copies of the K tile (the last ones may repeat a neighbour's: same bytes, same place)
+#pragma unroll
+        for (int i = 0; i < KPW; ++i) {
+            int inst = wave + i * NW;
+            inst = inst < KINSTR ? inst : KINSTR - 1;
+            const int pos = inst * 64 + lane;
+            const int row = pos / KCH;
+            const int logical = (pos % KCH) ^ swz_u<KCH>(row);
+            int grow = jt * BN + row;
+            grow = grow > n - 1 ? n - 1 : grow;
+            global_load_lds16(kbase + (int64_t)grow * k_rsb + logical * 16, smem + slot * KTILE + inst * 1024);
+        }
+        const char* src = dsrow + (int64_t)(2 * jt) * 2048 + lane * 16;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) global_load_lds16_nt(src + i * 1024, my_ds + slot * DSBYTES + i * 1024);
+    };
+
+    int ktr[2][DTK], krow_unused[DQK / 16];
+    lds_offsets_u<DQK>(krow_unused, ktr, lane);
+    // transposing reads of a stored block: lane (g, half, jrow, q4) supplies key 16 tt + 8 sec + 4 g + jrow, query rows
+    // 16 half + 4 q4 .. + 3, which sit in the 16 bytes of source lane (key, q4 & 1) of half `half`, upper 8 if q4 >= 2
+    int dtr[2][2];
+    {
+        const int i16 = lane & 15, half = (lane >> 4) & 1, jrow = i16 >> 2, q4 = i16 & 3;
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int sec = 0; sec < 2; ++sec) {
+                const int key = 16 * tt + 8 * sec + 4 * g + jrow;
+                dtr[tt][sec] = (64 * half + ((2 * key + (q4 & 1)) ^ (8 * half))) * 16 + (q4 >> 1) * 8;
+            }
+    }
+
+    f32x16_t dqacc[DTK][1];
+#pragma unroll
+    for (int dt = 0; dt < DTK; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dqacc[dt][0][r] = 0.f;
+
+    int t_cur = next_valid_tile<BN>(W, W.jt_begin);
+    int t_nxt = t_cur < jt_end ? next_valid_tile<BN>(W, t_cur + 1) : jt_end;
+    if (t_cur < jt_end) copy_step(t_cur, 0);
+    if (t_nxt < jt_end) copy_step(t_nxt, 1);
+    int slot = 0;
+    const bool has_targets = p.targets != nullptr;
+    while (t_cur < jt_end) {
+        // this tile has landed; the next one (if any) may still be in flight
+        if (t_nxt < jt_end) __builtin_amdgcn_s_waitcnt(0x0F70 | PER_STEP);
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();  // K of this tile is there for every wave, and nobody reads the tile before it any more
+        const int t_nn = t_nxt < jt_end ? next_valid_tile<BN>(W, t_nxt + 1) : jt_end;
+        if (t_nn < jt_end) copy_step(t_nn, slot == 0 ? 2 : slot - 1);
+        const char* kt = smem + slot * KTILE;
+        const char* dt_lds = my_ds + slot * DSBYTES;
+        const int S0 = (t_cur * BN) & ~(kKeyBlock - 1);
+        KeyBlockWalk walk;
+        walk.init(M, has_targets, S0, n);
+        const bool visited = wq0 < n && walk.visits(M, wq0 / kQueryTile, S0, n);
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub) {
+            const int s0 = t_cur * BN + sub * 32;
+            if (!visited || block_class32(M, !walk.scan, wq0, s0, n) == 0) continue;
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const vec8 dsT = read_vt_operand<TT>(dt_lds + sub * 2048 + dtr[tt][0], dt_lds + sub * 2048 + dtr[tt][1]);
+                const char* kb = kt + (sub * 32 + tt * 16) * KROW;
+#pragma unroll
+                for (int dt = 0; dt < DTK; ++dt)
+                    dqacc[dt][0] = TT::mfma(read_vt_operand<TT>(kb + ktr[0][dt], kb + ktr[1][dt]), dsT, dqacc[dt][0]);
+            }
+        }
+        t_cur = t_nxt;
+        t_nxt = t_nn;
+        slot = slot == 2 ? 0 : slot + 1;
+    }
+    store_output<TT, DTK>(dqacc, 0, bp.dq, W.seq_start, wq0 + l32, n, bp.dq_rs, bp.dq_hs, W.h, g, bp.gscale, DQK);
+}
+
 
 }  // namespace hstu

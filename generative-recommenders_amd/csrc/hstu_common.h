@@ -247,6 +247,13 @@ __device__ __forceinline__ void global_load_lds16(const char* src, const char* l
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(m0), "v"(src) : "memory");
 }
 
+// The same copy for data that is read once: marked non-temporal so that it does not displace what the other copies
+// of the kernel keep re-reading from L2.
+__device__ __forceinline__ void global_load_lds16_nt(const char* src, const char* lds_base) {
+    const unsigned m0 = (unsigned)(uintptr_t)HSTU_LDS(const char, lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" : : "s"(m0), "v"(src) : "memory");
+}
+
 // What one workgroup has to do; every field is wave-uniform.
 struct Work {
     int b, h;

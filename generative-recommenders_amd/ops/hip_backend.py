@@ -104,6 +104,7 @@ EXPORTS = (
     "hstu_hip_check_args",
     "hstu_hip_mha_fwd",
     "hstu_hip_mha_bwd",
+    "hstu_hip_mha_bwd_workspace_bytes",
     "hstu_hip_workspace_bytes",
     "hstu_hip_plan",
     "hstu_hip_tile_configs",
@@ -140,6 +141,8 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
         L.hstu_hip_mha_bwd.restype = ctypes.c_int
         L.hstu_hip_mha_bwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(HstuBwdGrads), ctypes.c_void_p]
+        L.hstu_hip_mha_bwd_workspace_bytes.restype = ctypes.c_size_t
+        L.hstu_hip_mha_bwd_workspace_bytes.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_plan.restype = ctypes.c_int
         L.hstu_hip_plan.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
         L.hstu_hip_workspace_bytes.restype = ctypes.c_size_t
@@ -291,6 +294,17 @@ def mha_fwd(
     raise_for_status(rc)
 
 
+def mha_bwd_workspace_bytes(total_rows: int, batch: int, heads: int, max_seq_len: int) -> int:
+    """Bytes of scratch with which ``mha_bwd`` stores dS instead of recomputing the scores for dq."""
+    a = HstuFwdArgs()
+    a.total_q, a.batch, a.heads, a.max_seq_len = total_rows, batch, heads, max_seq_len
+    return int(lib().hstu_hip_mha_bwd_workspace_bytes(ctypes.byref(a)))
+
+
+# Largest dS scratch mha_bwd takes by itself (the caching allocator keeps it between calls).
+BWD_SCRATCH_LIMIT_BYTES = 64 << 30
+
+
 def mha_bwd(
     dout: torch.Tensor,
     q: torch.Tensor,
@@ -307,9 +321,16 @@ def mha_bwd(
     contextual_seq_len: int,
     min_full_attn_seq_len: int,
     sort_by_length: bool = True,
+    store_ds: Optional[bool] = None,
+    workspace: Optional[torch.Tensor] = None,
 ) -> None:
     """Fill ``dq``, ``dk``, ``dv`` on the current stream of ``q.device`` (full attention only).  ``sort_by_length``
-    starts the long sequences first; it never changes the result."""
+    starts the long sequences first; it never changes the result.  ``store_ds``: let the kernel that forms dk and dv
+    write dS to scratch memory (2 bytes per query row, head and key position up to ``max_seq_len``) so that dq is one
+    streamed product instead of a second pass over the scores; ``None`` = when that scratch is at most
+    ``BWD_SCRATCH_LIMIT_BYTES`` and half of the device's free memory.  ``workspace``: the caller's own scratch (uint8,
+    256-byte aligned; ``mha_bwd_workspace_bytes`` says how much the stored form takes) instead of a fresh allocation;
+    it decides the form by its size."""
     a = HstuFwdArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), None
     a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
@@ -329,10 +350,24 @@ def mha_bwd(
     a.max_attn_len, a.contextual_seq_len, a.min_full_attn_seq_len = max_attn_len, contextual_seq_len, min_full_attn_seq_len
     a.dtype = _dtype_code(q.dtype)
     a.q_scale = a.k_scale = a.v_scale = 1.0
-    workspace = None
-    if sort_by_length and a.batch >= 2:
-        workspace = torch.empty(4 * a.batch, dtype=torch.uint8, device=q.device)
-        a.workspace, a.workspace_bytes, a.sort_by_length = workspace.data_ptr(), 4 * a.batch, 1
+    if workspace is not None:
+        torch._assert(workspace.dtype == torch.uint8 and workspace.is_contiguous() and workspace.device == q.device,
+                      "workspace must be a contiguous uint8 tensor on the inputs' device")
+        a.workspace, a.workspace_bytes = workspace.data_ptr(), workspace.numel()
+        a.sort_by_length = 1 if sort_by_length else 0
+    else:
+        need = 4 * a.batch if sort_by_length and a.batch >= 2 else 0
+        if store_ds is not False and a.total_q > 0 and a.batch > 0:
+            stored = lib().hstu_hip_mha_bwd_workspace_bytes(ctypes.byref(a))
+            if store_ds is None:
+                store_ds = stored <= BWD_SCRATCH_LIMIT_BYTES
+                if store_ds and not torch.cuda.is_current_stream_capturing():
+                    store_ds = 2 * stored <= torch.cuda.mem_get_info(q.device)[0]
+            if store_ds:
+                need = stored
+        if need:
+            workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+            a.workspace, a.workspace_bytes, a.sort_by_length = workspace.data_ptr(), need, 1 if sort_by_length else 0
     g = HstuBwdGrads()
     g.dout, g.dq, g.dk, g.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     g.do_row_stride, g.do_head_stride = dout.stride(0), dout.stride(1)

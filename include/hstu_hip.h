@@ -145,8 +145,18 @@ const char* hstu_hip_tile_config_name(int id);
  * written; no atomics, so the result is bit-identical from run to run.  The gradients have the layout rules of
  * q / k / v: 16-byte aligned base, row and head strides in elements and multiples of 8, innermost stride 1.
  * `sort_by_length` (a scheduling hint: long sequences first) takes effect when `args->workspace` holds at least
- * 4 * batch bytes; nothing else uses the workspace.
+ * 4 * batch bytes.
+ *
+ * Two ways to form dq.  Without more workspace than that, a second kernel recomputes the scores and dP from the query
+ * side (seven matrix products for the five the mathematics needs).  With a 256-byte aligned workspace of at least
+ * hstu_hip_mha_bwd_workspace_bytes(args) bytes -- 2 bytes per (query row, head, key position up to max_seq_len rounded
+ * up to 128), e.g. 17 GB for 128 sequences x 4096 rows x 4 heads -- the kernel that forms dk and dv also writes dS,
+ * rounded to the input type as the products use it, and dq is one streamed product dS K (HBM-bound; about a quarter
+ * less time in total).  The two differ only by the rounding of the pre-scaled operand (q or k) of the score product.
+ * The workspace need not be initialised and holds nothing of use afterwards.
  */
+size_t hstu_hip_mha_bwd_workspace_bytes(const HstuFwdArgs* args);
+
 typedef struct HstuBwdGrads {
     const void* dout;  /* [total_q, H, dv] */
     void* dq;          /* [total_q, H, dqk] */

@@ -126,12 +126,42 @@ def _run_bwd(pkg, dev, N, alpha, q, k, v, dout, offsets, offsets_dtype=torch.int
     return out.detach(), qd.grad, kd.grad, vd.grad
 
 
+def _direct(dev, N, alpha, q, k, v, dout, offsets, kw, **how):
+    """The backend's entry point without autograd; gradients pre-filled with a sentinel."""
+    from generative_recommenders_amd.ops import hip_backend
+
+    qd, kd, vd, dd, od = (t.to(dev) for t in (q, k, v, dout, offsets))
+    tg = kw.get("num_targets")
+    tg = None if tg is None else tg.to(dev)
+    dq, dk, dv = torch.full_like(qd, 7.0), torch.full_like(kd, 7.0), torch.full_like(vd, 7.0)
+    hip_backend.mha_bwd(dd, qd, kd, vd, dq, dk, dv, od, tg, N, alpha, kw.get("max_attn_len", 0), kw.get("contextual_seq_len", 0),
+                        kw.get("min_full_attn_seq_len", 0), **how)
+    torch.cuda.synchronize()
+    return dq, dk, dv
+
+
+def _poisoned_workspace(dev, q, offsets, N):
+    """Scratch for the stored-dS form with every 16-bit word a NaN: a block read without having been written shows."""
+    from generative_recommenders_amd.ops import hip_backend
+
+    need = hip_backend.mha_bwd_workspace_bytes(q.shape[0], offsets.numel() - 1, q.shape[1], N)
+    return torch.full((need,), 0xFF, dtype=torch.uint8, device=dev)
+
+
 def _check(pkg, dev, N, alpha, q, k, v, dout, offsets, what, **kw):
+    """Both forms of the backward against the closed form: dS stored (through autograd, and through the entry point on
+    NaN-filled scratch) and scores recomputed; dk and dv do not depend on the form."""
     out, dq, dk, dv = _run_bwd(pkg, dev, N, alpha, q, k, v, dout, offsets, **kw)
     rq, rk, rv = G.closed_form_grads(N, alpha, q, k, v, offsets, dout, **kw)
     _close(dq, rq, what + " dq")
     _close(dk, rk, what + " dk")
     _close(dv, rv, what + " dv")
+    if q.shape[0] > 0:
+        sq, sk, sv = _direct(dev, N, alpha, q, k, v, dout, offsets, kw, workspace=_poisoned_workspace(dev, q, offsets, N))
+        assert torch.equal(sq, dq) and torch.equal(sk, dk) and torch.equal(sv, dv), what + ": stored form on poisoned scratch"
+        cq, ck, cv = _direct(dev, N, alpha, q, k, v, dout, offsets, kw, store_ds=False)
+        _close(cq, rq, what + " dq recomputed")
+        assert torch.equal(ck, dk) and torch.equal(cv, dv), what + ": dk, dv of the two forms"
     return dq, dk, dv
 
 
@@ -208,25 +238,19 @@ VARIANT_CASES = [
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("store_ds", [False, True])
 @pytest.mark.parametrize("ci", range(len(VARIANT_CASES)))
-def test_backward_through_the_backend_entry_point(pkg, dev, ci):
+def test_backward_through_the_backend_entry_point(pkg, dev, ci, store_ds):
     """The backend's direct entry point (no autograd), gradients pre-filled with a sentinel: every row of every sequence
-    must be overwritten."""
-    from generative_recommenders_amd.ops import hip_backend
-
+    must be overwritten; both forms (scores recomputed for dq, or dS stored in NaN-filled scratch)."""
     lengths, H, dqk, dv, kw = VARIANT_CASES[ci]
-    print(f"[case] bwd direct {ci} {lengths}", flush=True)
+    print(f"[case] bwd direct {ci} {lengths} store_ds={store_ds}", flush=True)
     q, k, v, dout, offsets = _inputs(100 + ci, lengths, H, dqk, dv, torch.bfloat16)
     N, alpha = max(lengths) + 1, 1.0 / dqk**0.5
     ref = G.closed_form_grads(N, alpha, q, k, v, offsets, dout, **kw)
-    qd, kd, vd, dd, od = (t.to(dev) for t in (q, k, v, dout, offsets))
-    tg = kw.get("num_targets")
-    tg = None if tg is None else tg.to(dev)
-    dq, dk, dv_ = torch.full_like(qd, 7.0), torch.full_like(kd, 7.0), torch.full_like(vd, 7.0)
-    hip_backend.mha_bwd(dd, qd, kd, vd, dq, dk, dv_, od, tg, N, alpha, kw.get("max_attn_len", 0), kw.get("contextual_seq_len", 0),
-                        kw.get("min_full_attn_seq_len", 0))
-    torch.cuda.synchronize()
-    for name, x, r in zip(("dq", "dk", "dv"), (dq, dk, dv_), ref):
+    how = dict(workspace=_poisoned_workspace(dev, q, offsets, N)) if store_ds else dict(store_ds=False)
+    got = _direct(dev, N, alpha, q, k, v, dout, offsets, kw, **how)
+    for name, x, r in zip(("dq", "dk", "dv"), got, ref):
         _close(x, r, name)
 
 
@@ -242,13 +266,14 @@ def test_backward_of_a_long_sequence(pkg, dev):
 
 
 @pytest.mark.gpu
-def test_backward_at_the_size_of_the_ragged_benchmark(pkg, dev):
+@pytest.mark.parametrize("store_ds", [False, True])
+def test_backward_at_the_size_of_the_ragged_benchmark(pkg, dev, store_ds):
     """The third benchmark configuration (64 sequences up to 8192, window 2048, contextual prefix, targets): the
     longest and four other sequences against the closed form."""
     from generative_recommenders_amd import workloads
     from generative_recommenders_amd.ops import hip_backend
 
-    print("[case] bwd cfg3 full size", flush=True)
+    print(f"[case] bwd cfg3 full size store_ds={store_ds}", flush=True)
     wl = workloads.make_workload("cfg3")
     inp = workloads.make_inputs(wl, dev)
     q, k, v, offs, tg = inp["q"], inp["k"], inp["v"], inp["seq_offsets"], inp["num_targets"]
@@ -256,7 +281,7 @@ def test_backward_at_the_size_of_the_ragged_benchmark(pkg, dev):
     dout = (torch.randn(v.shape, device=dev, generator=g) * 0.1).to(v.dtype)
     dq, dk, dv = torch.full_like(q, 7.0), torch.full_like(k, 7.0), torch.full_like(v, 7.0)
     hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offs, tg, wl.max_seq_len, wl.alpha, wl.max_attn_len, wl.contextual_seq_len,
-                        wl.min_full_attn_seq_len)
+                        wl.min_full_attn_seq_len, store_ds=store_ds)
     torch.cuda.synchronize()
     order = sorted(range(wl.batch), key=lambda b: -int(wl.lengths[b]))
     picks = [order[0], order[7], order[20], order[40], order[63]]
@@ -271,12 +296,13 @@ def test_backward_at_the_size_of_the_ragged_benchmark(pkg, dev):
 
 
 @pytest.mark.gpu
-def test_backward_and_fused_producer_in_a_hip_graph(pkg, dev):
+@pytest.mark.parametrize("store_ds", [False, True])
+def test_backward_and_fused_producer_in_a_hip_graph(pkg, dev, store_ds):
     """hstu_compute_uqvk (fused kernel) -> hstu_mha forward -> backward kernels captured into one HIP graph: every
     replay, with eager work and a synchronisation in between, reproduces the eager results bit for bit."""
     from generative_recommenders_amd.ops import hip_backend, hstu_compute
 
-    print("[case] bwd + fused producer in a hip graph", flush=True)
+    print(f"[case] bwd + fused producer in a hip graph store_ds={store_ds}", flush=True)
     H, Dh, d_model = 2, 64, 256
     lengths = [700, 130, 1, 420]
     offsets = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int64).to(dev)
@@ -292,7 +318,7 @@ def test_backward_and_fused_producer_in_a_hip_graph(pkg, dev):
         u, q, k, v = hstu_compute.hstu_compute_uqvk(x, nw, nb, 1e-6, H, Dh, Dh, w, bias, path=2)
         out = pkg.hstu_mha(N, 0.125, q, k, v, offsets)
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)  # views' shapes, dense storage
-        hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offsets, None, N, 0.125, 0, 0, 0, sort_by_length=False)
+        hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offsets, None, N, 0.125, 0, 0, 0, sort_by_length=False, store_ds=store_ds)
         return out, dq, dk, dv
 
     with torch.no_grad():

@@ -75,6 +75,15 @@ def test_backward_argument_checks(backend):
     assert L.hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == -4
 
 
+def test_backward_workspace_bytes(backend):
+    """The dS scratch: 4 * batch bytes for the sequence order rounded up to 256, then (rows + 32 per sequence) x heads x
+    (max_seq_len rounded up to 128) x 2 bytes -- 17.3 GB at the size of the headline benchmark."""
+    assert backend.mha_bwd_workspace_bytes(100, 3, 2, 200) == 256 + (100 + 96) * 2 * 256 * 2
+    assert backend.mha_bwd_workspace_bytes(524288, 128, 4, 4096) == 512 + (524288 + 4096) * 4 * 4096 * 2
+    assert backend.mha_bwd_workspace_bytes(0, 3, 2, 200) == 0
+    assert backend.lib().hstu_hip_mha_bwd_workspace_bytes(None) == 0
+
+
 def test_jagged_copy_argument_checks(backend):
     """Validation of the jagged copy entry points runs before anything touches the device."""
     a = backend.HstuJaggedCopyArgs()
