@@ -10,19 +10,21 @@
 // P and dS are rounded to the operand type before their products, and the constant factors are applied to the fp32
 // sums at the end).  Nothing is saved by the forward pass: the scores are recomputed.
 //
-// Two kernels, each with the structure of the barrier-per-tile forward kernel (hstu_fwd_kernel.h) and without
-// atomics, so the result does not depend on the schedule:
+// Kernels, none with atomics, so the result does not depend on the schedule:
 //   * hstu_bwd_dkdv_kernel: a workgroup owns 128 key rows (K and V of 32 rows per wave in registers, K pre-scaled
 //     by c1 = -alpha * log2(e)) and walks the query rows that can see them in tiles of 64 (Q and dOut through LDS):
 //         S[q, kv]   = Q K^T          A = Q tile (row reads),            B = K registers
 //         dP[q, kv]  = dOut V^T       A = dOut tile (row reads),         B = V registers
 //         dV^T[dv, kv] += dOut^T P    A = dOut tile (transposing reads), B = P packed from the accumulator
 //         dK^T[d, kv]  += Q^T dS      A = Q tile (transposing reads),    B = dS packed
+//     On request it also writes every block of dS to scratch memory.
 //   * hstu_bwd_dq_kernel: a workgroup owns 128 query rows (Q pre-scaled and dOut in registers) and walks the key
 //     rows as the forward kernel does:
 //         S^T[kv, q]  = K Q^T         A = K tile (row reads),            B = Q registers
 //         dP^T[kv, q] = V dOut^T      A = V tile (row reads),            B = dOut registers
 //         dQ^T[d, q] += K^T dS^T      A = K tile (transposing reads),    B = dS^T packed
+//   * hstu_bwd_dq_stored_kernel, instead of the former when dS was stored: only the last of these three products, with
+//     dS^T read back from the scratch memory.
 // A tile that is read both by rows (ds_read_b128) and transposed (ds_read_b64_tr_b16) is stored with one chunk
 // swizzle that keeps both kinds of read off each other's banks (swz_u below).
 #pragma once
@@ -606,8 +608,9 @@ __global__ __launch_bounds__(NW * 64, 2) void hstu_bwd_dq_kernel(const BwdParams
 #pragma unroll
         for (int sub = 0; sub < BN / 32; ++sub) {
             const int s0 = jt * BN + sub * 32;  // first key row of the block of 32
+            // one instruction stream for every kind of block (see the key-stationary kernel): a block without a valid
+            // pair runs like the others and its dS is cleared afterwards
             const int cls = M.classify(wR0, wR1, s0, 32);
-            if (cls == 0) continue;
             f32x16_t s, dp;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
@@ -624,11 +627,28 @@ __global__ __launch_bounds__(NW * 64, 2) void hstu_bwd_dq_kernel(const BwdParams
                     const int r = half * 8 + j;
                     float pr, gr;
                     silu_and_slope(s[r], pr, gr);
-                    float dsr = dp[r] * gr;
-                    if (cls == 1) dsr = row.valid(M, s0 + 8 * (r >> 2) + 4 * g + (r & 3)) ? dsr : 0.f;
-                    d8[j] = dsr;
+                    d8[j] = dp[r] * gr;
                 }
                 dsb[half] = TT::pack8(d8);
+            }
+            if (cls != 2) {
+                typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    u32x4_t m;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        unsigned bits = 0;
+                        if (cls == 1) {
+                            const int r = 8 * half + 2 * w;
+                            const bool lo = row.valid(M, s0 + 8 * (r >> 2) + 4 * g + (r & 3));
+                            const bool hi = row.valid(M, s0 + 8 * ((r + 1) >> 2) + 4 * g + ((r + 1) & 3));
+                            bits = (lo ? 0xFFFFu : 0u) | (hi ? 0xFFFF0000u : 0u);
+                        }
+                        m[w] = bits;
+                    }
+                    dsb[half] = __builtin_bit_cast(vec8, __builtin_bit_cast(u32x4_t, dsb[half]) & m);
+                }
             }
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
