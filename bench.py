@@ -26,7 +26,7 @@ HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced ag
 # counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
 MEASURED_TRAFFIC_BYTES = {"headline": 2.414e9, "cfg2": 0.827e9, "cfg3": 1.383e9, "cfg4": 0.249e9, "cfg5": 2.281e9,
                           "kvcat": 0.173e9, "kvtail": 0.0168e9, "uqvk": 2.953e9, "layernorm": 1.074e9, "output": 5.839e9,
-                          "normmul": 2.684e9, "bwd": 6.284e9}
+                          "normmul": 2.684e9, "bwd": 6.246e9, "bwd_stored": 4.166e10}
 
 
 def run_gpu(wl, args, pkg, workloads, torch):
