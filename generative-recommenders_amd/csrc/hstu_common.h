@@ -540,22 +540,46 @@ __device__ __forceinline__ int next_valid_tile(const Work& w, int jt) {
     return jt;
 }
 
-// Per-lane constants of the mask predicate for one query row.
+// Per-lane constants of the mask predicate for one query row.  In key POSITIONS the predicate is a union of two
+// intervals and a point: ids are non-decreasing in the position, so "id(row) - w <= id(key) <= id(row) - 1" is
+// klo <= key <= khi, "contextual row and id(key) < max_id" is key < cend, and the row itself is always visible.
 struct RowMask {
     int pos;    // sequence position of the row
     int lo;     // id(row) - window: key ids in [lo, lo + w) pass the causal+window test
     int w;      // window of this row (INT_MAX if unlimited)
     bool ctx;   // contextual row: sees every non-target key
+    int klo, khi;  // first and last key position of the causal+window interval (khi = -1: empty)
+    int cend;      // keys before this position are visible to a contextual row (0 otherwise)
     __device__ __forceinline__ void init(const SeqMask& M, int row_pos) {
         const int idr = M.id(row_pos);
         pos = row_pos;
         w = (M.w == 0 || (M.f > 0 && idr >= M.max_id - M.f)) ? 0x7fffffff : M.w;
         lo = idr - w;
         ctx = M.c > 0 && idr == 0;
+        klo = lo > 0 ? lo + M.shift : 0;
+        khi = idr >= 1 ? idr - 1 + M.shift : -1;
+        cend = ctx ? M.max_id + M.shift : 0;
     }
     __device__ __forceinline__ bool valid(const SeqMask& M, int key_pos) const {
         const int ids = M.id(key_pos);
         return (key_pos == pos) | ((unsigned)(ids - lo) < (unsigned)w) | (ctx & (ids < M.max_id));
+    }
+    // Bit d = the key at position p0 + d is visible, d = 0 .. 31: the same predicate from the position intervals,
+    // about twenty operations for the 32 keys instead of a dozen per key.
+    __device__ __forceinline__ unsigned valid_bits(int p0) const {
+        auto upto = [](int b) -> unsigned {  // bits 0 .. b (none if b < 0, all if b >= 31)
+            const int bb = b > 31 ? 31 : (b < 0 ? 0 : b);
+            return b < 0 ? 0u : 0xFFFFFFFFu >> (31 - bb);
+        };
+        auto from = [](int a) -> unsigned {  // bits a .. 31 (all if a <= 0, none if a > 31)
+            const int aa = a < 0 ? 0 : (a > 31 ? 31 : a);
+            return a > 31 ? 0u : 0xFFFFFFFFu << aa;
+        };
+        const unsigned window = from(klo - p0) & upto(khi - p0);
+        const unsigned prefix = upto(cend - 1 - p0);
+        const int self = pos - p0;
+        const unsigned own = (unsigned)self < 32u ? 1u << (self & 31) : 0u;
+        return window | prefix | own;
     }
 };
 
@@ -570,6 +594,8 @@ template <class TT, int MASK>
 __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], float c1, const SeqMask& M,
                                           const RowMask& row, int sp0) {
     const int causal_room = row.pos - sp0;  // a key at offset d from sp0 is visible iff d <= causal_room
+    unsigned bits = 0;
+    if (MASK == 1) bits = row.valid_bits(sp0);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         // eight elements at a time, fenced, so that the scheduler cannot pile up temporaries of all sixteen
@@ -578,7 +604,8 @@ __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (
         for (int j = 0; j < 8; ++j) {
             const int r = half * 8 + j;
             float pr = TT::silu(s[r], c1);
-            if (MASK == 1) pr = row.valid(M, sp0 + 8 * (r >> 2) + (r & 3)) ? pr : 0.f;
+            if (MASK == 1)  // all ones or zero from the key's bit, AND-ed onto the value
+                pr = __builtin_bit_cast(float, __builtin_bit_cast(int, pr) & __builtin_amdgcn_sbfe((int)bits, 8 * (r >> 2) + (r & 3), 1));
             if (MASK == 2) pr = (8 * (r >> 2) + (r & 3) <= causal_room) ? pr : 0.f;
             p[j] = pr;
         }

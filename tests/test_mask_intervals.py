@@ -1,0 +1,49 @@
+"""The kernels evaluate the mask of a masked tile per query row as a union of two intervals of key POSITIONS and a
+point (RowMask::valid_bits in csrc/hstu_common.h).  This test restates that form in Python and checks it against the
+reference's id formula (oracle.get_valid_attn_mask, ops/pytorch/pt_hstu_attention.py:32-84) by brute force over every
+small setting: sequence length, number of targets, window, contextual prefix, min_full_attn_seq_len."""
+
+import itertools
+
+import torch
+
+from oracle import hstu_oracle
+
+
+def _interval_mask(n, targets, w, c, f):
+    """valid[row, key] from the per-row constants the kernel keeps: klo, khi, cend, pos."""
+    shift = c - 1 if c > 0 else 0
+    max_id = n - (targets or 0) - shift
+
+    def ident(pos):  # ids are clamped to max_id only when targets are given
+        x = max(pos - shift, 0)
+        return x if targets is None else min(x, max_id)
+
+    valid = torch.zeros((n, n), dtype=torch.bool)
+    for row in range(n):
+        idr = ident(row)
+        wr = 0x7FFFFFFF if (w == 0 or (f > 0 and idr >= max_id - f)) else w
+        lo = idr - wr
+        ctx = c > 0 and idr == 0
+        klo = lo + shift if lo > 0 else 0
+        khi = idr - 1 + shift if idr >= 1 else -1
+        cend = max_id + shift if ctx else 0
+        for key in range(n):
+            valid[row, key] = (key == row) or (klo <= key <= khi) or (key < cend)
+    return valid
+
+
+def test_position_intervals_equal_the_id_formula():
+    checked = 0
+    for n, c, w, f in itertools.product([1, 2, 5, 9, 14], [0, 1, 3, 6], [0, 1, 2, 4, 20], [0, 2, 5]):
+        if f > 0 and w == 0:
+            continue
+        for targets in [None] + list(range(0, n + 1)):
+            if c > 0 and n - (targets or 0) < c:
+                continue  # the reference asserts that the contextual prefix fits into the non-target part
+            lengths = torch.tensor([n])
+            want = hstu_oracle.get_valid_attn_mask(True, n, lengths, None if targets is None else torch.tensor([targets]), w, c, f)[0]
+            got = _interval_mask(n, targets, w, c, f)
+            assert torch.equal(got, want), (n, targets, w, c, f)
+            checked += 1
+    assert checked > 1000
