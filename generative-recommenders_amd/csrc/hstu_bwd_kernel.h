@@ -221,12 +221,28 @@ __device__ __forceinline__ void silu_and_slope(float t, float& p, float& g) {
 
 // ---- key-stationary kernel: dK, dV ---------------------------------------------------------------------------------
 
-// Per-lane constants of the mask predicate for one key.
+// Per-lane constants of the mask predicate for one key.  In row POSITIONS the rows that see a key are a union of
+// intervals and a point (ids are non-decreasing in the position): [rlo, rhi] from "id(key) + 1 <= id(row) <= id(key) + w",
+// [r2lo, n) for the rows whose window min_full_attn_seq_len lifts, [0, crows) for the contextual rows, and the key's own
+// row.
 struct KeyMask {
     int pos, ids;
+    int rlo, rhi, r2lo, crows;
     __device__ __forceinline__ void init(const SeqMask& M, int key_pos) {
+        constexpr int kNone = 1 << 30;
         pos = key_pos;
         ids = M.id(key_pos);
+        const bool clamped = M.idclamp != 0x7fffffff;  // targets given: ids stop at max_id
+        rlo = (clamped && ids + 1 > M.max_id) ? kNone : ids + 1 + M.shift;
+        const int w = M.w < kNone ? M.w : kNone;
+        rhi = (M.w == 0 || (clamped && ids + w >= M.max_id)) ? kNone : ids + w + M.shift;
+        r2lo = kNone;
+        if (M.w > 0 && M.f > 0) {
+            const int first_full = M.max_id - M.f;
+            const int r2 = first_full <= 0 ? 0 : first_full + M.shift;
+            r2lo = r2 > rlo ? r2 : rlo;
+        }
+        crows = (M.c > 0 && ids < M.max_id) ? M.shift + 1 : 0;
     }
     // rows at or past the end of the sequence are padding of the last tile
     __device__ __forceinline__ bool valid(const SeqMask& M, int row_pos) const {
@@ -234,6 +250,21 @@ struct KeyMask {
         const int wr = (M.w == 0 || (M.f > 0 && idr >= M.max_id - M.f)) ? 0x7fffffff : M.w;
         const bool ok = (row_pos == pos) | ((unsigned)(idr - ids - 1) < (unsigned)wr) | ((M.c > 0) & (idr == 0) & (ids < M.max_id));
         return ok & (row_pos < M.n);
+    }
+    // Bit d = the row at position p0 + d sees this key, d = 0 .. 31 (the same predicate from the intervals).
+    __device__ __forceinline__ unsigned valid_bits(int p0, int n) const {
+        auto upto = [](int b) -> unsigned {  // bits 0 .. b (none if b < 0, all if b >= 31)
+            const int bb = b > 31 ? 31 : (b < 0 ? 0 : b);
+            return b < 0 ? 0u : 0xFFFFFFFFu >> (31 - bb);
+        };
+        auto from = [](int a) -> unsigned {  // bits a .. 31 (all if a <= 0, none if a > 31)
+            const int aa = a < 0 ? 0 : (a > 31 ? 31 : a);
+            return a > 31 ? 0u : 0xFFFFFFFFu << aa;
+        };
+        const int self = pos - p0;
+        const unsigned own = (unsigned)self < 32u ? 1u << (self & 31) : 0u;
+        const unsigned m = (from(rlo - p0) & upto(rhi - p0)) | from(r2lo - p0) | upto(crows - 1 - p0) | own;
+        return m & upto(n - 1 - p0);
     }
 };
 
@@ -449,19 +480,16 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
     typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
     auto apply_mask = [&](int cls, int r0, vec8 (&pb_o)[2], vec8 (&dsb_o)[2]) __attribute__((always_inline)) {
         if (cls == 2) return;
+        const unsigned rows = cls == 1 ? key.valid_bits(r0 + 4 * g, n) : 0u;  // bit d: row r0 + 4 g + d sees the lane's key
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             u32x4_t m;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                unsigned bits = 0;
-                if (cls == 1) {
-                    const int e = 8 * h + 2 * w;
-                    const bool lo = key.valid(M, r0 + 8 * (e >> 2) + 4 * g + (e & 3));
-                    const bool hi = key.valid(M, r0 + 8 * ((e + 1) >> 2) + 4 * g + ((e + 1) & 3));
-                    bits = (lo ? 0xFFFFu : 0u) | (hi ? 0xFFFF0000u : 0u);
-                }
-                m[w] = bits;
+                const int e = 8 * h + 2 * w, d = 8 * (e >> 2) + (e & 3);  // elements e, e + 1: rows d, d + 1
+                const unsigned lo = (unsigned)__builtin_amdgcn_sbfe((int)rows, d, 1);
+                const unsigned hi = (unsigned)__builtin_amdgcn_sbfe((int)rows, d + 1, 1);
+                m[w] = (lo & 0xFFFFu) | (hi & 0xFFFF0000u);
             }
             pb_o[h] = __builtin_bit_cast(vec8, __builtin_bit_cast(u32x4_t, pb_o[h]) & m);
             dsb_o[h] = __builtin_bit_cast(vec8, __builtin_bit_cast(u32x4_t, dsb_o[h]) & m);
@@ -634,18 +662,16 @@ __global__ __launch_bounds__(NW * 64, 2) void hstu_bwd_dq_kernel(const BwdParams
             if (cls != 2) {
                 typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
 #pragma unroll
+                const unsigned keys = cls == 1 ? row.valid_bits(s0 + 4 * g) : 0u;  // bit d: key s0 + 4 g + d is visible
+#pragma unroll
                 for (int half = 0; half < 2; ++half) {
                     u32x4_t m;
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
-                        unsigned bits = 0;
-                        if (cls == 1) {
-                            const int r = 8 * half + 2 * w;
-                            const bool lo = row.valid(M, s0 + 8 * (r >> 2) + 4 * g + (r & 3));
-                            const bool hi = row.valid(M, s0 + 8 * ((r + 1) >> 2) + 4 * g + ((r + 1) & 3));
-                            bits = (lo ? 0xFFFFu : 0u) | (hi ? 0xFFFF0000u : 0u);
-                        }
-                        m[w] = bits;
+                        const int r = 8 * half + 2 * w, d = 8 * (r >> 2) + (r & 3);  // elements r, r + 1: keys d, d + 1
+                        const unsigned lo = (unsigned)__builtin_amdgcn_sbfe((int)keys, d, 1);
+                        const unsigned hi = (unsigned)__builtin_amdgcn_sbfe((int)keys, d + 1, 1);
+                        m[w] = (lo & 0xFFFFu) | (hi & 0xFFFF0000u);
                     }
                     dsb[half] = __builtin_bit_cast(vec8, __builtin_bit_cast(u32x4_t, dsb[half]) & m);
                 }

@@ -33,6 +33,37 @@ def _interval_mask(n, targets, w, c, f):
     return valid
 
 
+def _column_interval_mask(n, targets, w, c, f):
+    """The same matrix from the per-KEY constants of the backward (KeyMask in csrc/hstu_bwd_kernel.h): the rows that see
+    key k are [rlo, rhi], [r2lo, n) (rows whose window is lifted by min_full_attn_seq_len), [0, crows) (contextual
+    rows) and k itself."""
+    big = 1 << 30
+    shift = c - 1 if c > 0 else 0
+    max_id = n - (targets or 0) - shift
+
+    def ident(pos):
+        x = max(pos - shift, 0)
+        return x if targets is None else min(x, max_id)
+
+    valid = torch.zeros((n, n), dtype=torch.bool)
+    for key in range(n):
+        ids = ident(key)
+        clamped = targets is not None
+        rlo = big if (clamped and ids + 1 > max_id) else ids + 1 + shift
+        if w == 0:
+            rhi = big
+        else:
+            rhi = big if (clamped and ids + w >= max_id) else ids + w + shift
+        r2lo = big
+        if w > 0 and f > 0:
+            first_full = max_id - f
+            r2lo = max(rlo, 0 if first_full <= 0 else first_full + shift)
+        crows = shift + 1 if (c > 0 and ids < max_id) else 0
+        for row in range(n):
+            valid[row, key] = (row == key) or (rlo <= row <= rhi) or (row >= r2lo) or (row < crows)
+    return valid
+
+
 def test_position_intervals_equal_the_id_formula():
     checked = 0
     for n, c, w, f in itertools.product([1, 2, 5, 9, 14], [0, 1, 3, 6], [0, 1, 2, 4, 20], [0, 2, 5]):
@@ -45,5 +76,6 @@ def test_position_intervals_equal_the_id_formula():
             want = hstu_oracle.get_valid_attn_mask(True, n, lengths, None if targets is None else torch.tensor([targets]), w, c, f)[0]
             got = _interval_mask(n, targets, w, c, f)
             assert torch.equal(got, want), (n, targets, w, c, f)
+            assert torch.equal(_column_interval_mask(n, targets, w, c, f), want), ("per key", n, targets, w, c, f)
             checked += 1
     assert checked > 1000
