@@ -661,7 +661,6 @@ __global__ __launch_bounds__(NW * 64, 2) void hstu_bwd_dq_kernel(const BwdParams
             }
             if (cls != 2) {
                 typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
-#pragma unroll
                 const unsigned keys = cls == 1 ? row.valid_bits(s0 + 4 * g) : 0u;  // bit d: key s0 + 4 g + d is visible
 #pragma unroll
                 for (int half = 0; half < 2; ++half) {

@@ -558,7 +558,7 @@ struct RowMask {
         ctx = M.c > 0 && idr == 0;
         klo = lo > 0 ? lo + M.shift : 0;
         khi = idr >= 1 ? idr - 1 + M.shift : -1;
-        cend = ctx ? M.max_id + M.shift : 0;
+        cend = (ctx && M.max_id > 0) ? M.max_id + M.shift : 0;  // a sequence shorter than the prefix has max_id <= 0: nothing passes
     }
     __device__ __forceinline__ bool valid(const SeqMask& M, int key_pos) const {
         const int ids = M.id(key_pos);

@@ -7,6 +7,7 @@
 #include <hipblaslt/hipblaslt.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 #include <tuple>
@@ -302,11 +303,17 @@ int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hi
 constexpr size_t kGemmScratch = 64u << 20;
 enum GemmEpilogue { kEpiNone = 0, kEpiBias = 1, kEpiBiasSilu = 2 };
 
+constexpr int kGemmCandidates = 16;
+
 struct GemmPlan {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr, d = nullptr;
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
+    // the library's other proposals for this problem, until one call has timed them (see gemm())
+    hipblasLtMatmulHeuristicResult_t candidates[kGemmCandidates];
+    int ncandidates = 0;
+    bool tuned = false;
 };
 
 struct GemmShape {
@@ -364,13 +371,13 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
         if ((st = hipblasLtMatmulPreferenceCreate(&pref)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("preference", st);
         const uint64_t max_ws = kGemmScratch;
         hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
-        hipblasLtMatmulHeuristicResult_t res[1];
         int found = 0;
-        st = hipblasLtMatmulAlgoGetHeuristic(g_handle, pl.desc, pl.a, pl.b, pl.c, pl.d, pref, 1, res, &found);
+        st = hipblasLtMatmulAlgoGetHeuristic(g_handle, pl.desc, pl.a, pl.b, pl.c, pl.d, pref, kGemmCandidates, pl.candidates, &found);
         hipblasLtMatmulPreferenceDestroy(pref);
         if (st != HIPBLAS_STATUS_SUCCESS || found < 1) return blaslt_fail("hipblasLtMatmulAlgoGetHeuristic", st);
-        pl.algo = res[0].algo;
-        pl.workspace = res[0].workspaceSize;
+        pl.ncandidates = found;
+        pl.algo = pl.candidates[0].algo;
+        pl.workspace = pl.candidates[0].workspaceSize;
         it = g_plans.emplace(key, pl).first;
     }
     GemmPlan& pl = it->second;
@@ -379,6 +386,45 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
         if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("bias pointer", st);
     }
     const float one = 1.0f, beta = residual ? 1.0f : 0.0f;
+    // The library's first proposal is not always its fastest for these shapes (shallow products of half a million rows).
+    // The first call that may do so times every proposal on the caller's own operands (as the reference's Triton kernels
+    // autotune on first use) and keeps the fastest; every proposal computes the same product, so `out` ends up right
+    // whichever ran last.  Not while the stream is being captured into a graph (events cannot be waited for), and not
+    // when the product accumulates onto its own output.
+    if (!pl.tuned && pl.ncandidates > 1 && getenv("HSTU_LINEAR_NO_TUNING") == nullptr) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        const bool capturing = hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
+        if (!capturing && residual != out) {
+            hipEvent_t e0 = nullptr, e1 = nullptr;
+            if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+                float best = 0.f;
+                int best_i = -1;
+                for (int i = 0; i < pl.ncandidates; ++i) {
+                    if (pl.candidates[i].workspaceSize > kGemmScratch) continue;
+                    float fastest = 0.f;
+                    bool ok = true;
+                    for (int rep = 0; rep < 3 && ok; ++rep) {
+                        (void)hipEventRecord(e0, stream);
+                        st = hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out,
+                                             pl.d, &pl.candidates[i].algo, scratch, pl.candidates[i].workspaceSize, stream);
+                        (void)hipEventRecord(e1, stream);
+                        float ms = 0.f;
+                        ok = st == HIPBLAS_STATUS_SUCCESS && hipEventSynchronize(e1) == hipSuccess &&
+                             hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+                        if (ok && rep > 0 && (fastest == 0.f || ms < fastest)) fastest = ms;  // the first run warms up
+                    }
+                    if (ok && fastest > 0.f && (best_i < 0 || fastest < best)) best = fastest, best_i = i;
+                }
+                if (best_i >= 0) {
+                    pl.algo = pl.candidates[best_i].algo;
+                    pl.workspace = pl.candidates[best_i].workspaceSize;
+                }
+                pl.tuned = true;
+            }
+            if (e0) (void)hipEventDestroy(e0);
+            if (e1) (void)hipEventDestroy(e1);
+        }
+    }
     st = hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out, pl.d, &pl.algo,
                          scratch, pl.workspace, stream);
     if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmul", st);

@@ -133,6 +133,8 @@ EDGE = [
     ("window_eq_tile", [300, 150], [7, 3], 320, 64, 0, 0),
     ("window_gt_len", [100, 90], [7, 3], 128, 1000, 3, 0),
     ("ctx_only_prefix", [40, 300], None, 320, 0, 40, 0),
+    ("ctx_longer_than_sequences", [30, 300, 59, 61], None, 320, 0, 60, 0),
+    ("ctx_longer_than_non_targets", [90, 200, 70], [50, 150, 69], 256, 9, 60, 0),
     ("ctx_targets_window", [500, 131, 260], [100, 1, 130], 512, 37, 6, 0),
     ("ctx_big_window_small", [700, 300], [30, 200], 1024, 3, 130, 0),
     ("min_full", [400, 150, 90], [20, 0, 5], 400, 16, 4, 24),
