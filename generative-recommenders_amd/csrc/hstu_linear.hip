@@ -386,24 +386,30 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
         if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("bias pointer", st);
     }
     const float one = 1.0f, beta = residual ? 1.0f : 0.0f;
-    // The library's first proposal is not always its fastest for these shapes (shallow products of half a million rows).
-    // The first call that may do so times every proposal on the caller's own operands (as the reference's Triton kernels
-    // autotune on first use) and keeps the fastest; every proposal computes the same product, so `out` ends up right
-    // whichever ran last.  Not while the stream is being captured into a graph (events cannot be waited for), and not
-    // when the product accumulates onto its own output.
-    if (!pl.tuned && pl.ncandidates > 1 && getenv("HSTU_LINEAR_NO_TUNING") == nullptr) {
+    // With HSTU_LINEAR_TUNING=1 in the environment the first call that may do so times every proposal of the library on the
+    // caller's own operands (as the reference's Triton kernels autotune on first use) and keeps the fastest if it beats the
+    // library's first choice by 3 %; every proposal computes the same product, so `out` ends up right whichever ran last.
+    // Off by default: measured on the two shapes of the benchmark, the proposals lie within +-4 % of each other and the
+    // winner of a back-to-back timing is not reliably the winner between the other kernels of a layer (-6 % for the
+    // v|q|k product, +2 % for the output projection).  Never while the stream is being captured into a graph (events
+    // cannot be waited for), and not when the product accumulates onto its own output.
+    if (!pl.tuned && pl.ncandidates > 1 && getenv("HSTU_LINEAR_TUNING") != nullptr) {
         hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
         const bool capturing = hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone;
         if (!capturing && residual != out) {
             hipEvent_t e0 = nullptr, e1 = nullptr;
             if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
-                float best = 0.f;
+                float best = 0.f, first = 0.f;
                 int best_i = -1;
+                // bring the clocks and the caches to where a running loop has them before anything is timed
+                for (int rep = 0; rep < 8; ++rep)
+                    (void)hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out,
+                                          pl.d, &pl.candidates[0].algo, scratch, pl.candidates[0].workspaceSize, stream);
                 for (int i = 0; i < pl.ncandidates; ++i) {
                     if (pl.candidates[i].workspaceSize > kGemmScratch) continue;
                     float fastest = 0.f;
                     bool ok = true;
-                    for (int rep = 0; rep < 3 && ok; ++rep) {
+                    for (int rep = 0; rep < 5 && ok; ++rep) {
                         (void)hipEventRecord(e0, stream);
                         st = hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out,
                                              pl.d, &pl.candidates[i].algo, scratch, pl.candidates[i].workspaceSize, stream);
@@ -413,8 +419,11 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
                              hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
                         if (ok && rep > 0 && (fastest == 0.f || ms < fastest)) fastest = ms;  // the first run warms up
                     }
+                    if (ok && i == 0) first = fastest;
                     if (ok && fastest > 0.f && (best_i < 0 || fastest < best)) best = fastest, best_i = i;
                 }
+                // the library's own first choice stays unless another one is clearly (3 %) faster
+                if (best_i > 0 && first > 0.f && best > 0.97f * first) best_i = 0;
                 if (best_i >= 0) {
                     pl.algo = pl.candidates[best_i].algo;
                     pl.workspace = pl.candidates[best_i].workspaceSize;

@@ -178,6 +178,25 @@ def test_compute_output(pkg, dev, N, H, ld, D, cu, cx, act, group_norm, dtype):
 
 
 @pytest.mark.gpu
+def test_output_with_the_library_proposals_timed(pkg, dev, monkeypatch):
+    """HSTU_LINEAR_TUNING=1: the first call of a new shape runs every proposal of the GEMM library; the result is the same
+    product, and later calls (one of them with the switch off again) reproduce it bit for bit."""
+    print("[case] output with HSTU_LINEAR_TUNING", flush=True)
+    N, H, ld, D = 2304, 2, 64, 192  # a shape no other test uses, so the plan is made here
+    attn, u, x, nw, nb, w = _inputs(4242, N, H, ld, D, 3, False, torch.bfloat16)
+    args = [t.to(dev) for t in (attn, u, x, nw, nb)] + [1e-6, w.to(dev), H, ld, 0.0, False, True, True, "silu", False, False]
+    monkeypatch.setenv("HSTU_LINEAR_TUNING", "1")
+    first = pkg.hstu_compute_output(*args)
+    again = pkg.hstu_compute_output(*args)
+    monkeypatch.delenv("HSTU_LINEAR_TUNING")
+    later = pkg.hstu_compute_output(*args)
+    torch.cuda.synchronize()
+    kw = dict(concat_u=True, concat_x=True, mul_u_activation_type="silu", group_norm=False, num_heads=H, linear_dim=ld)
+    _close(first, O.compute_output(attn, u, x, nw, nb, w, 1e-6, **kw), "tuned out vs fp32 oracle")
+    assert torch.equal(first, again) and torch.equal(first, later)
+
+
+@pytest.mark.gpu
 def test_output_takes_strided_views_and_rejects_what_it_cannot_do(pkg, dev):
     N, H, ld, D = 50, 2, 64, 64
     attn, u, x, nw, nb, w = [t.to(dev) for t in _inputs(5, N, H, ld, D, 3, False, torch.bfloat16)]
