@@ -271,7 +271,7 @@ def run_linear(name, args, pkg, torch):
     print(json.dumps(line))
 
 
-def run_bwd(name, args, pkg, workloads, torch):
+def run_bwd(name, args, pkg, workloads, torch, emit=True):
     """Backward of hstu_mha (dq, dk, dv from dout) on the headline shape (`bwd`) or on the ragged third baseline
     configuration (`bwd_cfg3`).  A step is one call of the backward entry point: its two kernels.  Algorithmic work:
     five products per mask-valid pair (S, dP, dV, dQ, dK -- the count of the reference's bench,
@@ -322,7 +322,7 @@ def run_bwd(name, args, pkg, workloads, torch):
                      "kernel_ms": round(ev_ms, 4),
                      "algorithmic_flops": flops, "algorithmic_bytes": nbytes},
     }
-    if not args.no_cpu:
+    if not args.no_cpu and emit:
         cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
         torch.set_num_threads(cores)
         order = sorted(range(wl.batch), key=lambda b: -int(wl.lengths[b]))
@@ -347,7 +347,9 @@ def run_bwd(name, args, pkg, workloads, torch):
         line["cpu_baseline"] = {"value": round(cpu_flops / t_used / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                                 "sample": f"{len(done)} of {wl.batch} sequences (lengths {[int(wl.lengths[b]) for b in done]}), "
                                           f"fp32 closed-form gradients per sequence, {t_used:.1f} s"}
-    print(json.dumps(line))
+    if emit:
+        print(json.dumps(line))
+    return line
 
 
 def main():
@@ -367,6 +369,8 @@ def main():
                     help="HBM-priced workloads (cfg2, cfg4, kvcat, kvtail): do not flush the caches between steps")
     ap.add_argument("--no-jagged", action="store_true",
                     help="headline only: do not also time the ragged cfg3 batch for the extra `jagged_cfg3` entry")
+    ap.add_argument("--no-bwd", action="store_true",
+                    help="headline only: do not also time the backward of the same call for the extra `backward` entry")
     ap.add_argument("--no-sort", action="store_true", help="do not pass sort_by_length=True to hstu_mha")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 1 GiB device copy, so that a counter run can scale FETCH_SIZE/WRITE_SIZE")
@@ -471,6 +475,16 @@ def main():
             "note": "reference convention = H*(Dqk+Dv)*sum(n^2), the figure the reference's bench prints; it counts pairs "
                     "that max_attn_len masks out",
         }
+    if wl.name == "headline" and not args.no_bwd:
+        # the backward of the same call (dq, dk, dv from dout), measured in the same run: about half a second
+        saved = (args.steps, args.warmup)
+        args.steps, args.warmup = 10, 3
+        b = run_bwd("bwd", args, pkg, workloads, torch, emit=False)
+        args.steps, args.warmup = saved
+        line["backward"] = {"workload": "bwd", "form": b["config"]["form"], "scratch_bytes": b["config"]["scratch_bytes"],
+                            "kernel_ms": b["roofline"]["kernel_ms"], "exact_tflops": b["value"], "pct_mfma_peak": b["pct_mfma_peak"],
+                            "kernels": b["roofline"]["kernel"],
+                            "note": "2 * (3 * Dqk + 2 * Dv) flops per mask-valid pair, the count of the reference's bench"}
     if not args.no_cpu:
         line["cpu_baseline"] = run_cpu_baseline(wl, torch, workloads)
     print(json.dumps(line))
