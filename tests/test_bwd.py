@@ -296,6 +296,42 @@ def test_backward_at_the_size_of_the_ragged_benchmark(pkg, dev, store_ds):
 
 
 @pytest.mark.gpu
+def test_backward_forms_agree_at_the_size_of_the_headline_benchmark(pkg, dev):
+    """64 sequences of 8192 rows, 4 heads of 128: the dS scratch is 34.5 GB, so its addresses need all of their 64 bits.
+    dk and dv of the two forms are the same bits; dq differs only by the rounding of the pre-scaled operand; one
+    sequence is also checked against the closed form."""
+    from generative_recommenders_amd import workloads
+    from generative_recommenders_amd.ops import hip_backend
+
+    print("[case] bwd headline size, both forms", flush=True)
+    wl = workloads.make_workload("headline")
+    inp = workloads.make_inputs(wl, dev)
+    q, k, v, offs = inp["q"], inp["k"], inp["v"], inp["seq_offsets"]
+    g = torch.Generator(device=dev).manual_seed(78)
+    dout = (torch.randn(v.shape, device=dev, generator=g) * 0.1).to(v.dtype)
+    need = hip_backend.mha_bwd_workspace_bytes(q.shape[0], wl.batch, wl.heads, wl.max_seq_len)
+    if 2 * need > torch.cuda.mem_get_info(dev)[0]:
+        pytest.skip("not enough free device memory for the scratch")
+    got = {}
+    for form in ("stored", "recompute"):
+        dq, dk, dv = torch.full_like(q, 7.0), torch.full_like(k, 7.0), torch.full_like(v, 7.0)
+        scratch = torch.full((need,), 0xFF, dtype=torch.uint8, device=dev) if form == "stored" else None
+        hip_backend.mha_bwd(dout, q, k, v, dq, dk, dv, offs, None, wl.max_seq_len, wl.alpha, 0, 0, 0, store_ds=False, workspace=scratch)
+        torch.cuda.synchronize()
+        del scratch
+        got[form] = (dq, dk, dv)
+    assert torch.equal(got["stored"][1], got["recompute"][1]) and torch.equal(got["stored"][2], got["recompute"][2])
+    a, b = got["stored"][0].float(), got["recompute"][0].float()
+    assert torch.isfinite(a).all()
+    assert float((a - b).norm() / b.norm()) <= 5e-3
+    last = wl.batch - 1  # the sequence whose blocks lie at the far end of the scratch
+    ref = G.closed_form_grads(wl.max_seq_len, wl.alpha, q.cpu(), k.cpu(), v.cpu(), offs.cpu(), dout.cpu(), sequences=[last])
+    s0, s1 = int(offs[last]), int(offs[last + 1])
+    for name, x, r in zip(("dq", "dk", "dv"), got["stored"], ref):
+        _close(x[s0:s1], r[s0:s1], f"headline size, last sequence, {name}")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("store_ds", [False, True])
 def test_backward_and_fused_producer_in_a_hip_graph(pkg, dev, store_ds):
     """hstu_compute_uqvk (fused kernel) -> hstu_mha forward -> backward kernels captured into one HIP graph: every
