@@ -302,7 +302,7 @@ def mha_bwd_workspace_bytes(total_rows: int, batch: int, heads: int, max_seq_len
 
 
 # Largest dS scratch mha_bwd takes by itself (the caching allocator keeps it between calls).
-BWD_SCRATCH_LIMIT_BYTES = 64 << 30
+BWD_SCRATCH_LIMIT_BYTES = 40 << 30
 
 
 def mha_bwd(
