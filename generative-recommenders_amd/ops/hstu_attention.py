@@ -6,10 +6,10 @@ messages and output shapes.  Differences, all explicit:
 
 * there is one backend, so ``kernel`` / ``enable_tma`` are accepted and ignored; ``sort_by_length`` is, as in
   the reference, a scheduling hint (long sequences are started first) that never changes the result;
-* ``hstu_mha`` is differentiable for bf16 / fp16 inputs (``dq, dk, dv`` come from the backward kernels through an
-  autograd function, as ``_AttentionFunction`` does in the reference, ``triton_hstu_attention.py:2978-3093``);
-  ``delta_hstu_mha`` and the fp32 / fp8 forms are forward only -- inputs that require grad under
-  ``torch.enable_grad()`` raise ``NotImplementedError`` there;
+* ``hstu_mha`` is differentiable for bf16 / fp16 / fp32 inputs (``dq, dk, dv`` come from the backward kernels through
+  an autograd function, as ``_AttentionFunction`` does in the reference, ``triton_hstu_attention.py:2978-3093``; for
+  fp32 inputs the backward runs on bf16 copies and widens its results); ``delta_hstu_mha`` and the fp8 form are
+  forward only -- inputs that require grad under ``torch.enable_grad()`` raise ``NotImplementedError`` there;
 * tensors must live on a HIP device; there is no CPU or PyTorch fallback;
 * fp32 q/k/v are rounded to fp16 inside the library (11-bit significand; the reference's Triton path multiplies in
   tf32) and give an fp32 result;
@@ -75,14 +75,22 @@ class _HstuMhaFunction(torch.autograd.Function):
         q, k, v, seq_offsets = ctx.saved_tensors[:4]
         num_targets = ctx.saved_tensors[4] if ctx.has_targets else None
         max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len = ctx.params
+        # fp32 inputs: the backward kernels take 16-bit operands, so they run on bf16 copies (fp32's range, 8 bits of
+        # mantissa; the products accumulate in fp32 as always) and the gradients are widened again -- the counterpart
+        # of the forward's fp16 copies, with the range of dout, which can be tiny, kept whole
+        wide = q.dtype == torch.float32
+        if wide:
+            q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
         # rows of sequences longer than max_seq_len are outside the contract and get no gradient
         dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
         if q.numel() > 0:
-            dout = _kernel_layout(dout.detach())
+            dout = _kernel_layout(dout.detach().to(q.dtype))
             hip_backend.mha_bwd(
                 dout, q, k, v, dq, dk, dv, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
                 min_full_attn_seq_len,
             )
+        if wide:
+            dq, dk, dv = dq.float(), dk.float(), dv.float()
         return (dq, dk, dv) + (None,) * 10
 
 
@@ -139,7 +147,7 @@ def hstu_mha(
         num_targets = _index_tensor(num_targets, "num_targets")
     seq_offsets = _index_tensor(seq_offsets, "seq_offsets")
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
-        if q.dtype not in (torch.bfloat16, torch.float16):
+        if q.dtype not in (torch.bfloat16, torch.float16, torch.float32):
             _check_forward_only(q, k, v)
         return _HstuMhaFunction.apply(
             q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len,

@@ -380,10 +380,31 @@ def test_backward_and_fused_producer_in_a_hip_graph(pkg, dev, store_ds):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("mi", [0, 4])
+def test_backward_of_fp32_inputs(pkg, dev, mi):
+    """fp32 is the second dtype of the reference's own test grid (hstu_attention_test.py:271-275).  The kernels take
+    16-bit operands: the forward runs on fp16 copies, the backward on bf16 copies (dout can be tiny), both accumulate in
+    fp32 and return fp32.  Bar: the bf16 one (relative Frobenius <= 1e-2, max-abs <= 2e-2 max|ref|) against the closed
+    form evaluated on the fp32 inputs themselves."""
+    print(f"[case] bwd fp32 inputs mask={mi}", flush=True)
+    lengths = [300, 129, 1, 64]
+    q, k, v, dout, offsets = _inputs(31 + mi, lengths, 2, 64, 64, torch.float32)
+    mask = {a: (int(b * 20) if isinstance(b, int) and not isinstance(b, bool) else b) for a, b in MASKS[mi].items()}
+    kw = _mask_kwargs(mask, lengths, 7)
+    out, dq, dk, dv = _run_bwd(pkg, dev, 320, 0.125, q, k, v, dout * 1e-4, offsets, **kw)  # small upstream gradients
+    assert out.dtype == torch.float32 and dq.dtype == torch.float32 and dk.dtype == torch.float32 and dv.dtype == torch.float32
+    rq, rk, rv = G.closed_form_grads(320, 0.125, q, k, v, offsets, dout * 1e-4, **kw)
+    _close(dq, rq, "fp32 dq")
+    _close(dk, rk, "fp32 dk")
+    _close(dv, rv, "fp32 dv")
+
+
+@pytest.mark.gpu
 def test_backward_rejections(pkg, dev):
     q, k, v, dout, offsets = _inputs(1, [40, 24], 2, 32, 32, torch.float32)
-    with pytest.raises(NotImplementedError):
-        pkg.hstu_mha(64, 0.2, q.to(dev).requires_grad_(), k.to(dev), v.to(dev), offsets.to(dev))
+    with pytest.raises(NotImplementedError):  # fp8 inputs have no backward
+        pkg.hstu_mha(64, 0.2, q.to(torch.float8_e4m3fn).to(dev).requires_grad_(), k.to(torch.float8_e4m3fn).to(dev),
+                     v.to(torch.float8_e4m3fn).to(dev), offsets.to(dev))
     with pytest.raises(NotImplementedError):
         pkg.delta_hstu_mha(64, 0.2, q.bfloat16()[:16].to(dev).requires_grad_(), k.bfloat16().to(dev), v.bfloat16().to(dev), offsets.to(dev))
     # no gradient asked for: the plain forward path, no graph

@@ -528,11 +528,11 @@ def test_wrapper_rejects_what_it_cannot_do(pkg, dev):
         pkg.hstu_mha(32, 0.1, q.double().to(dev), k.double().to(dev), v.double().to(dev), offs.to(dev))
     with pytest.raises(NotImplementedError):  # fp32 runs on the generic kernel only
         pkg.hstu_mha(32, 0.1, q.float().to(dev), k.float().to(dev), v.float().to(dev), offs.to(dev), tile_config=2)
-    qg = q.float().to(dev).requires_grad_()  # the backward exists for bf16 / fp16 only
+    qg = _quantize(q)[0].to(dev).requires_grad_()  # no backward for fp8 inputs
     with pytest.raises(NotImplementedError):
-        pkg.hstu_mha(32, 0.1, qg, k.float().to(dev), v.float().to(dev), offs.to(dev))
+        pkg.hstu_mha(32, 0.1, qg, _quantize(k)[0].to(dev), _quantize(v)[0].to(dev), offs.to(dev))
     with torch.no_grad():
-        pkg.hstu_mha(32, 0.1, qg, k.float().to(dev), v.float().to(dev), offs.to(dev))
+        pkg.hstu_mha(32, 0.1, qg, _quantize(k)[0].to(dev), _quantize(v)[0].to(dev), offs.to(dev))
     torch.cuda.synchronize()
 
 
