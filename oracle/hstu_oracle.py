@@ -258,6 +258,7 @@ def hstu_mha_per_sequence(
     row_chunk: int = 1024,
     compute_dtype: torch.dtype = torch.float32,
     sequences: Optional[list] = None,
+    row_ranges: Optional[list] = None,
 ) -> torch.Tensor:
     """Same mathematics as PT:129-251, one sequence at a time at its own length.
 
@@ -265,6 +266,8 @@ def hstu_mha_per_sequence(
     ``delta_size > 0``: ``q`` is ``[B * delta_size, H, Dqk]`` holding the last
     ``delta_size`` positions of each sequence; the result is ``[B * delta_size, H, Dv]``.
     ``sequences`` restricts the work to those batch indices (other rows stay zero).
+    ``row_ranges`` (a list of ``(r0, r1)`` in query-row indices of a sequence, clipped to its rows) restricts it
+    further to those query rows; a row's result does not depend on which other rows are evaluated with it.
     """
     H = q.shape[1]
     V = v.shape[2]
@@ -285,8 +288,9 @@ def hstu_mha_per_sequence(
         else:
             rows0, q0 = 0, s0
             nq = n
-        for c0 in range(0, nq, row_chunk):
-            c1 = min(nq, c0 + row_chunk)
+        spans = [(0, nq)] if row_ranges is None else [(max(0, a), min(nq, z)) for a, z in row_ranges]
+        chunks = [(c0, min(z, c0 + row_chunk)) for a, z in spans for c0 in range(a, z, row_chunk)]
+        for c0, c1 in chunks:
             qb = q[q0 + c0 : q0 + c1].to(compute_dtype).transpose(0, 1)  # [H, m, D]
             s = torch.matmul(qb, kb.transpose(1, 2)) * alpha
             s = F.silu(s) / max_seq_len

@@ -497,6 +497,79 @@ def test_cfg3_shape_subset(pkg, dev):
         assert_parity(got[s0:s1], ref[s0:s1], f"cfg3 seq {b} n={s1 - s0}")
 
 
+@pytest.mark.parametrize("sort", [False, True])
+def test_headline_shape_subset(pkg, dev, sort):
+    """The shape of the headline benchmark at full size (B=64 sequences of 8192 rows, H=4, d=128, bf16, causal), with
+    the kernel and schedule the library picks by itself (equal lengths: the strided deal of the 256-row kernel);
+    `sort` is the hint the benchmark passes.  Oracle on whole sequences: the first, the last and two in between."""
+    from generative_recommenders_amd import workloads
+
+    wl = workloads.make_workload("headline")
+    _announce("headline full size", wl.total_kv, "sort_by_length", sort)
+    g = torch.Generator(device=dev).manual_seed(wl.seed)
+    q, k, v = [(torch.randn((wl.total_kv, wl.heads, wl.dqk), device=dev, generator=g) * 0.1).to(torch.bfloat16) for _ in range(3)]
+    offs = torch.arange(wl.batch + 1, dtype=torch.int64) * wl.max_seq_len
+    got = pkg.hstu_mha(wl.max_seq_len, wl.alpha, q, k, v, offs.to(dev), sort_by_length=sort)
+    torch.cuda.synchronize()
+    from generative_recommenders_amd.ops import hip_backend
+
+    assert hip_backend.plan_for(wl.batch, wl.heads, wl.dqk, wl.dv, wl.total_kv, wl.total_kv, wl.max_seq_len, sort_by_length=sort) == (2, 1)
+    for b in (0, 21, 42, 63):
+        s0, s1 = b * wl.max_seq_len, (b + 1) * wl.max_seq_len
+        ref = _ref_full(q[s0:s1].cpu(), k[s0:s1].cpu(), v[s0:s1].cpu(), torch.tensor([0, s1 - s0]), None, wl.max_seq_len, wl.alpha)
+        assert_parity(got[s0:s1], ref, f"headline seq {b}")
+
+
+def test_cfg5_shape_subset(pkg, dev):
+    """Baseline config 5 at full size: e4m3 q/k/v quantised per tensor from absmax exactly as the benchmark does it,
+    B=16, lengths 4096..16384, H=8, d=128, N=16384, targets.  Cosine >= 0.995 against the oracle on the un-quantised
+    inputs (the stated bar) and >= 0.998 against the oracle on the de-quantised ones, on every row of the shortest
+    and of a middle sequence, on the first, a middle and the last rows of the longest, and on the last 512 rows of
+    every sequence (those hold all the targets); the generic kernel, written independently, on all rows."""
+    from generative_recommenders_amd import workloads
+
+    wl = workloads.make_workload("cfg5")
+    inp = workloads.make_inputs(wl, torch.device("cpu"))
+    _announce("cfg5 full size", wl.total_kv)
+    q, k, v, offs, t = inp["q"], inp["k"], inp["v"], inp["seq_offsets"], inp["num_targets"]
+    (qq, qs), (kq, ks), (vq, vs) = _quantize(q), _quantize(k), _quantize(v)
+    kw = dict(num_targets=t.to(dev), q_scale=qs, k_scale=ks, v_scale=vs)
+    args = (wl.max_seq_len, wl.alpha, qq.to(dev), kq.to(dev), vq.to(dev), offs.to(dev))
+    got = pkg.hstu_mha(*args, sort_by_length=True, **kw)
+    other = pkg.hstu_mha(*args, tile_config=1, **kw)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and torch.isfinite(got.float()).all()
+    from generative_recommenders_amd.ops import hip_backend
+
+    assert hip_backend.plan_for(wl.batch, wl.heads, wl.dqk, wl.dv, wl.total_kv, wl.total_kv, wl.max_seq_len, sort_by_length=True,
+                                dtype=hip_backend.HSTU_FP8_E4M3) == (2, 1)
+    assert _cos(got.cpu(), other.cpu()) >= 0.9995
+    assert_parity(got, other.float(), "cfg5: ping-pong kernel vs generic kernel", rel_tol=3e-2)
+    got = got.cpu()
+    deq = (qq.float() * qs, kq.float() * ks, vq.float() * vs)
+    order = np.argsort(wl.lengths)
+    lo, mid, hi = int(order[0]), int(order[len(order) // 2]), int(order[-1])
+    n_hi = int(wl.lengths[hi])
+
+    def check(what, rows, **sel):
+        ref = _ref_full(q, k, v, offs, t, wl.max_seq_len, wl.alpha, **sel)[rows]
+        ref_q = _ref_full(*deq, offs, t, wl.max_seq_len, wl.alpha, **sel)[rows]
+        cos, cos_q = _cos(got[rows], ref), _cos(got[rows], ref_q)
+        assert cos >= 0.995, f"cfg5 {what}: cosine vs un-quantised oracle {cos:.5f}"
+        assert cos_q >= 0.998, f"cfg5 {what}: cosine vs de-quantised oracle {cos_q:.5f}"
+
+    for b in (lo, mid):
+        check(f"seq {b} n={int(wl.lengths[b])}", slice(int(offs[b]), int(offs[b + 1])), sequences=[b])
+    spans = [(0, 512), (n_hi // 2, n_hi // 2 + 512), (n_hi - 1024, n_hi)]
+    rows = torch.cat([torch.arange(int(offs[hi]) + a, int(offs[hi]) + z) for a, z in spans])
+    check(f"longest seq {hi} n={n_hi}", rows, sequences=[hi], row_ranges=spans)
+    tails = torch.cat([torch.arange(int(offs[b + 1]) - 512, int(offs[b + 1])) for b in range(wl.batch)])
+    for name, src in (("un-quantised", (q, k, v)), ("de-quantised", deq)):
+        ref = O.cached_hstu_mha_per_sequence(wl.max_seq_len, wl.alpha, src[0][tails].float(), src[1].float(), src[2].float(), offs, t)
+        cos = _cos(got[tails], ref)
+        assert cos >= (0.995 if name == "un-quantised" else 0.998), f"cfg5 tail rows vs {name} oracle: cosine {cos:.5f}"
+
+
 def test_cfg4_shape_subset(pkg, dev):
     """Baseline config 4 (M-FALCON: 32 users, history 1024..4096, 256 delta queries) at full size."""
     from generative_recommenders_amd import workloads

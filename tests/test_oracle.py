@@ -117,6 +117,18 @@ def test_dense_oracle_matches_scalar_c(case):
         row_chunk=17,
     )
     torch.testing.assert_close(per_seq, ref, atol=1e-7, rtol=1e-4)
+    # restricted to some query rows: those rows as in the scalar checker's result, every other row untouched
+    spans = [(0, 3), (7, 19), (28, 1000)]
+    some = O.hstu_mha_per_sequence(
+        N, alpha, q, k, v, offs, num_targets=t, max_attn_len=w, contextual_seq_len=c, min_full_attn_seq_len=f,
+        row_chunk=5, row_ranges=spans,
+    )
+    keep = torch.zeros(q.shape[0], dtype=torch.bool)
+    for b in range(len(lengths)):
+        for a, z in spans:
+            keep[int(offs[b]) + a : min(int(offs[b]) + z, int(offs[b + 1]))] = True
+    torch.testing.assert_close(some[keep], ref[keep], atol=1e-7, rtol=1e-4)
+    assert not some[~keep].any()
 
 
 @pytest.mark.parametrize("delta,w,c", [(8, 0, 0), (5, 6, 2), (1, 0, 3)])
