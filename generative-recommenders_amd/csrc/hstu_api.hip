@@ -12,6 +12,12 @@
 #include "hstu_fwd_pp_kernel.h"
 #include "hstu_jagged_kernels.h"
 
+// Scratch area of hstu_hip_mha_fwd_noalloc: what the caller's `workspace` is to hstu_hip_mha_fwd (work-item counters,
+// sequence ranking, work lists, partial sums of a kv-split), held by every device the library is loaded on until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress: the device address it yields (one
+// per device) is what kernels and copies are given.  Its size, HSTU_NOALLOC_SCRATCH_BYTES, is part of the interface.
+static __device__ __align__(256) unsigned char scratch[HSTU_NOALLOC_SCRATCH_BYTES];
+
 namespace hstu {
 
 // Work done ahead of the forward kernel, in the caller's workspace (either part may be absent):
@@ -306,6 +312,7 @@ const char* hstu_hip_status_string(int status) {
         case HSTU_ERR_UNSUPPORTED: return "argument combination not built";
         case HSTU_ERR_LAUNCH: return "HIP launch failed";
         case HSTU_ERR_BAD_DEVICE: return "current device is not gfx950";
+        case HSTU_ERR_SCRATCH_LIMIT: return "the call needs more scratch memory than the library's fixed area holds";
         default: return "unknown status";
     }
 }
@@ -518,6 +525,51 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
     if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
     return launch_dim<hstu::Fp8>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
+}
+
+namespace {
+
+// Device address of `scratch` on the current device (each device holds its own copy of the array at its own address),
+// looked up once per device with that device current; NULL if the lookup fails.
+void* noalloc_scratch_of_current_device() {
+    static void* cache[64];  // racing threads store the same value
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    if (!cache[dev]) {
+        void* ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            set_last_error("hipGetSymbolAddress(scratch)", e);
+            return nullptr;
+        }
+        cache[dev] = ptr;
+    }
+    return cache[dev];
+}
+
+}  // namespace
+
+int hstu_hip_mha_fwd_noalloc(const HstuFwdArgs* a, void* stream) {
+    g_last_error[0] = 0;
+    int rc = hstu_hip_check_args(a);
+    if (rc != HSTU_OK) return rc;
+    if (a->total_q == 0 || a->batch == 0) return HSTU_OK;
+    if (!current_device_is_gfx950()) return HSTU_ERR_BAD_DEVICE;
+    const size_t need = make_plan(a).total();
+    if (need > (size_t)HSTU_NOALLOC_SCRATCH_BYTES) {
+        snprintf(g_last_error, sizeof(g_last_error), "this call would use %zu bytes of scratch memory; the fixed area holds %zu", need,
+                 (size_t)HSTU_NOALLOC_SCRATCH_BYTES);
+        return HSTU_ERR_SCRATCH_LIMIT;
+    }
+    void* ptr = noalloc_scratch_of_current_device();
+    if (!ptr) return HSTU_ERR_LAUNCH;
+    HstuFwdArgs b = *a;
+    b.workspace = ptr;  // the device address, never the array's name
+    b.workspace_bytes = (int64_t)HSTU_NOALLOC_SCRATCH_BYTES;
+    // Everything the kernels read from the area is written earlier in the same call (counters and ranking by the prep
+    // kernel, work lists by the plan kernel, run counts and partial sums by the forward kernel), so what an earlier
+    // call left behind is never looked at and nothing has to be cleared.
+    return hstu_hip_mha_fwd(&b, stream);
 }
 
 }  // extern "C"

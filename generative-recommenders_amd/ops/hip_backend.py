@@ -103,6 +103,7 @@ EXPORTS = (
     "hstu_hip_last_error",
     "hstu_hip_check_args",
     "hstu_hip_mha_fwd",
+    "hstu_hip_mha_fwd_noalloc",
     "hstu_hip_mha_bwd",
     "hstu_hip_mha_bwd_workspace_bytes",
     "hstu_hip_workspace_bytes",
@@ -139,6 +140,8 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_check_args.argtypes = [ctypes.POINTER(HstuFwdArgs)]
         L.hstu_hip_mha_fwd.restype = ctypes.c_int
         L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
+        L.hstu_hip_mha_fwd_noalloc.restype = ctypes.c_int
+        L.hstu_hip_mha_fwd_noalloc.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
         L.hstu_hip_mha_bwd.restype = ctypes.c_int
         L.hstu_hip_mha_bwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(HstuBwdGrads), ctypes.c_void_p]
         L.hstu_hip_mha_bwd_workspace_bytes.restype = ctypes.c_size_t
@@ -172,6 +175,7 @@ _STATUS_EXC = {
     -6: NotImplementedError,
     -7: RuntimeError,
     -8: RuntimeError,
+    -9: RuntimeError,
 }
 
 
@@ -244,11 +248,14 @@ def mha_fwd(
     sort_by_length: bool = False,
     kv_splits: int = 0,
     workspace_bytes: Optional[int] = None,
+    noalloc: bool = False,
 ) -> None:
     """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors.
 
     ``workspace_bytes``: scratch to hand to the library; ``None`` = as much as it asks for.  With less it skips
-    the scheduling options that do not fit (the result is the same)."""
+    the scheduling options that do not fit (the result is the same).
+    ``noalloc``: go through ``hstu_hip_mha_fwd_noalloc``, which keeps its scratch in a fixed area inside the library
+    instead (no allocation here or there; calls that overlap in time on one device must not use it together)."""
     a = HstuFwdArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
@@ -283,6 +290,12 @@ def mha_fwd(
     need = lib().hstu_hip_workspace_bytes(ctypes.byref(a))
     if workspace_bytes is not None:
         need = min(need, workspace_bytes)
+    if noalloc:
+        with torch.cuda.device(q.device):
+            stream = torch.cuda.current_stream(q.device).cuda_stream
+            rc = lib().hstu_hip_mha_fwd_noalloc(ctypes.byref(a), ctypes.c_void_p(stream))
+        raise_for_status(rc)
+        return
     if need > 0:
         # scratch for the schedule; the caching allocator keeps it alive until the stream has consumed it
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)

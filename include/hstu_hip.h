@@ -41,7 +41,8 @@ enum HstuStatus {
     HSTU_ERR_BAD_SHAPE = -5,      /* negative / inconsistent sizes, max_seq_len <= 0, delta rows not B*delta */
     HSTU_ERR_UNSUPPORTED = -6,    /* legal in the reference but not built here */
     HSTU_ERR_LAUNCH = -7,         /* hipLaunchKernel failed; see hstu_hip_last_error() */
-    HSTU_ERR_BAD_DEVICE = -8      /* the current device is not gfx950 */
+    HSTU_ERR_BAD_DEVICE = -8,     /* the current device is not gfx950 */
+    HSTU_ERR_SCRATCH_LIMIT = -9   /* hstu_hip_mha_fwd_noalloc: the call needs more than HSTU_NOALLOC_SCRATCH_BYTES */
 };
 
 /*
@@ -115,6 +116,26 @@ int hstu_hip_check_args(const HstuFwdArgs* args);
  * delta-query (M-FALCON) forms.
  */
 int hstu_hip_mha_fwd(const HstuFwdArgs* args, void* stream);
+
+/*
+ * The same forward pass for callers that cannot allocate device memory: code under HIP graph capture, serving loops
+ * with a fixed memory budget, harnesses that forbid hipMalloc.  No counterpart in the reference (its native op
+ * allocates its tile semaphore and output itself, flash_common.cpp:596-678).  `args->workspace` is ignored: the scratch
+ * memory hstu_hip_mha_fwd would take from it (work-item counters, sequence ranking, work lists, partial sums of a
+ * kv-split) lives in a fixed area of HSTU_NOALLOC_SCRATCH_BYTES inside the library's device image, one per device,
+ * held until the process ends.  The call allocates and frees nothing, on the device or through any library; the
+ * caller still passes q, k, v, out and the index arrays.  Same kernels, same schedule and bit-identical results as
+ * hstu_hip_mha_fwd given a workspace of hstu_hip_workspace_bytes(args).
+ * Returns HSTU_ERR_SCRATCH_LIMIT (nothing launched; hstu_hip_last_error() names the two sizes) when
+ * hstu_hip_workspace_bytes(args) exceeds the area -- FP32 inputs of more than a few million elements (their fp16
+ * copies live there), kv-splits of very large delta batches, work lists of more than about 6 million row blocks.
+ * All calls on one device share that device's area: two calls that may run at the same time on one device (different
+ * streams, or different threads) race on it and must be serialised by the caller; calls on one stream are safe back
+ * to back.  Nothing needs clearing between calls (every word a kernel reads was written earlier in the same call).
+ * The first call on a device looks the area's address up (hipGetSymbolAddress); make that call outside a capture.
+ */
+#define HSTU_NOALLOC_SCRATCH_BYTES (48u << 20)
+int hstu_hip_mha_fwd_noalloc(const HstuFwdArgs* args, void* stream);
 
 /*
  * Bytes of `workspace` the call would use with these arguments (0 if it needs none).  The library never
