@@ -13,6 +13,7 @@ from .common import HammerKernel  # noqa: F401
 from .ops.hstu_attention import delta_hstu_mha, hstu_mha  # noqa: F401
 from .ops.hstu_compute import hstu_compute_output, hstu_compute_uqvk, hstu_preprocess_and_attention  # noqa: F401
 from .ops.jagged_tensors import concat_2D_jagged, split_2D_jagged, write_kv_tail  # noqa: F401
+from .ops import native_op  # noqa: F401  (defines torch.ops.hstu.hstu_mha / hstu_mha_fwd on these kernels)
 
 __all__ = [
     "HammerKernel", "hstu_mha", "delta_hstu_mha", "concat_2D_jagged", "split_2D_jagged", "write_kv_tail", "hstu_compute_uqvk",

@@ -49,6 +49,33 @@ __global__ __launch_bounds__(256) void hstu_prep_kernel(const void* offsets, int
     if (lane == 0) order[rank] = i;
 }
 
+// The caller contract checked on the device: report[0] = number of sequences that break it, report[1] = the first
+// such sequence, report[2] = what it breaks (bit 0: offsets decrease, 1: longer than max_seq_len, 2: num_targets outside
+// [0, length], 3: fewer non-target positions than contextual_seq_len, 4: shorter than delta_size), report[3] = 1 if
+// seq_offsets[0] != 0 or seq_offsets[batch] != total_kv.  One thread per sequence.
+__global__ __launch_bounds__(256) void hstu_check_contract_kernel(const void* offsets, int offsets_i64, const void* targets, int targets_i64,
+                                                                   int B, long long total_kv, int max_seq_len, int c, int delta,
+                                                                   int* report) {
+    auto off = [&](int j) -> long long { return offsets_i64 ? ((const long long*)offsets)[j] : (long long)((const int*)offsets)[j]; };
+    const int b = blockIdx.x * 256 + threadIdx.x;
+    if (b == 0 && (off(0) != 0 || off(B) != total_kv)) report[3] = 1;
+    if (b >= B) return;
+    const long long n = off(b + 1) - off(b);
+    long long t = 0;
+    if (targets) t = targets_i64 ? ((const long long*)targets)[b] : (long long)((const int*)targets)[b];
+    int what = 0;
+    if (n < 0) what |= 1;
+    if (n > max_seq_len) what |= 2;
+    if (t < 0 || t > n) what |= 4;
+    if (n > 0 && n - t < c) what |= 8;
+    if (delta > 0 && n < delta) what |= 16;
+    if (what) {
+        atomicAdd(report, 1);
+        atomicMin(report + 1, b);
+        atomicOr(report + 2, what);
+    }
+}
+
 }  // namespace hstu
 
 namespace {
@@ -353,6 +380,8 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     if (a->tile_config < 0 || a->tile_config > kNumConfigs) return HSTU_ERR_BAD_SHAPE;
     if (a->kv_splits < 0 || a->kv_splits > kMaxSplits || (a->kv_splits > 1 && a->tile_config == 1)) return HSTU_ERR_BAD_SHAPE;
     if (a->workspace && (a->workspace_bytes < 0 || (reinterpret_cast<uintptr_t>(a->workspace) & 3) != 0)) return HSTU_ERR_MISALIGNED;
+    if (a->attn_scale && (reinterpret_cast<uintptr_t>(a->attn_scale) & 3) != 0) return HSTU_ERR_MISALIGNED;
+    if (a->attn_scale && a->delta_size > 0) return HSTU_ERR_UNSUPPORTED;  // the reference's cached form has no attn_scale
     // head dims 16 / 32 / 64 / 128, independently for q/k and v (the grid of the reference's tests,
     // hstu_attention_test.py:266-267; its native op wants them equal, flash_common.cpp:543-545); 8-bit rows are at
     // least 32 wide
@@ -371,6 +400,31 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
     const int64_t out_mask = a->dtype == HSTU_FP32 ? 3 : 7;
     for (int i = 0; i < 8; ++i)
         if (strides[i] < 0 || (strides[i] & (i < 6 ? in_mask : out_mask)) != 0) return HSTU_ERR_MISALIGNED;
+    return HSTU_OK;
+}
+
+int hstu_hip_check_contract(const HstuFwdArgs* a, int32_t* report, void* stream_) {
+    g_last_error[0] = 0;
+    int rc = hstu_hip_check_args(a);
+    if (rc != HSTU_OK) return rc;
+    if (!report) return HSTU_ERR_NULL_POINTER;
+    hipStream_t stream = (hipStream_t)stream_;
+    // a small fill kernel would do as well; this memset is outside anything a caller captures (the check reads back)
+    const int32_t init[4] = {0, 0x7fffffff, 0, 0};
+    hipError_t e = hipMemcpyAsync(report, init, sizeof(init), hipMemcpyHostToDevice, stream);
+    if (e != hipSuccess) {
+        set_last_error("hipMemcpyAsync", e);
+        return HSTU_ERR_LAUNCH;
+    }
+    if (a->batch == 0 || !a->seq_offsets) return HSTU_OK;
+    hipLaunchKernelGGL(hstu::hstu_check_contract_kernel, dim3((a->batch + 255) / 256), dim3(256), 0, stream, a->seq_offsets,
+                       a->seq_offsets_i64, a->num_targets, a->num_targets_i64, a->batch, (long long)a->total_kv, a->max_seq_len,
+                       a->contextual_seq_len, a->delta_size, report);
+    e = hipGetLastError();
+    if (e != hipSuccess) {
+        set_last_error("contract kernel launch", e);
+        return HSTU_ERR_LAUNCH;
+    }
     return HSTU_OK;
 }
 
@@ -409,11 +463,15 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     p.f = a->min_full_attn_seq_len;
     p.c1 = -a->alpha * 1.4426950408889634f;
     p.oscale = a->alpha == 0.0f ? 0.0f : -1.0f / ((float)a->max_seq_len * 1.4426950408889634f);
+    p.oscale_unit = a->alpha == 0.0f ? 0.0f : -1.0f / 1.4426950408889634f;
+    p.attn_scale = (const float*)a->attn_scale;
+    p.attn_scale_per_row = a->attn_scale_per_row;
     if (a->dtype == HSTU_FP8_E4M3) {
         // real value = stored value * scale: the score scales go into c1 (applied to the accumulator), the
         // value scale and the factor P is stored with go into the output scale
         p.c1 *= a->q_scale * a->k_scale;
         p.oscale *= a->v_scale / hstu::Fp8::PSCALE;
+        p.oscale_unit *= a->v_scale / hstu::Fp8::PSCALE;
     }
 
     // Every use of the caller's scratch memory is an optimisation that never changes the result: without enough of

@@ -75,6 +75,11 @@ struct FwdParams {
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
     float c1;           // -alpha * log2(e): Q is multiplied by it when loaded
     float oscale;       // (alpha / max_seq_len) / c1 = -1 / (max_seq_len * log2(e)); 0 if alpha == 0
+    // attn_scale of the reference (pt_hstu_attention.py:152-165): a factor per query row, or one for all, that takes the
+    // place of 1 / max_seq_len.  NULL = none; `oscale_unit` is `oscale` without the 1 / max_seq_len.
+    const float* attn_scale;
+    int attn_scale_per_row;
+    float oscale_unit;
     // Split of the kv range of a row block into runs of `kv_chunk` tiles, each taken by its own workgroup; the
     // grid holds `kv_splits` workgroups per row block (1 = off) and those past the end of a short range exit at
     // once.  Each run writes its unscaled fp32 accumulators to partial[split][row][head][dv] (dense) and run 0
@@ -699,6 +704,12 @@ __device__ __forceinline__ typename TT::vec8 read_vt_operand(const char* lo_addr
     }
 }
 
+// The factor the fp32 accumulators of output row `row` (index into out, clamped by the caller) are multiplied with.
+__device__ __forceinline__ float output_scale(const FwdParams& p, int64_t row) {
+    if (!p.attn_scale) return p.oscale;
+    return p.oscale_unit * p.attn_scale[p.attn_scale_per_row ? row : 0];
+}
+
 // out[q, dv] = oscale * O^T[dv, q] for one block of 32 query rows; the lane holds 4 consecutive dv per
 // (dv tile, r/4), stored as 8 bytes.  QT is deduced from the accumulator array.
 template <class TT, int DT, int QT>
@@ -837,8 +848,9 @@ __global__ __launch_bounds__(256) void hstu_reduce_splits_kernel(const FwdParams
         acc += x;
     }
     elem4 o4;
+    const float osc = output_scale(p, row);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o4[i] = (ELEM)(acc[i] * p.oscale);
+    for (int i = 0; i < 4; ++i) o4[i] = (ELEM)(acc[i] * osc);
     *(elem4*)(p.o + (row * p.o_rs + (int64_t)h * p.o_hs) * 2 + c * 8) = o4;
 }
 

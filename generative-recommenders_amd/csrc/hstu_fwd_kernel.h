@@ -136,7 +136,10 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
 
     const int64_t orow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) store_output<TT, DT>(oacc, qt, p.o, orow0, wq0 + qt * 32 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale, DV);
+    for (int qt = 0; qt < QT; ++qt) {
+        const int ql = wq0 + qt * 32 + l32;
+        store_output<TT, DT>(oacc, qt, p.o, orow0, ql, nq, p.o_rs, p.o_hs, W.h, g, output_scale(p, orow0 + (ql < nq ? ql : nq - 1)), DV);
+    }
 }
 
 }  // namespace hstu

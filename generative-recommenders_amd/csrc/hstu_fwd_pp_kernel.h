@@ -484,10 +484,11 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         // tile around in its own piece of that LDS
         __syncthreads();
         store_output_via_lds<TT, DT>(oacc, smem + wave * (32 * (DT * 64 + 16)), p.o, orow0, wq0, nq, p.o_rs, p.o_hs, W.h,
-                                     lane, p.oscale);
+                                     lane, output_scale(p, orow0 + (wq0 + l32 < nq ? wq0 + l32 : nq - 1)));
     } else {
         // 8-bit K/V tiles are smaller than the 16-bit output staging would be
-        store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g, p.oscale);
+        store_output<TT, DT>(oacc, 0, p.o, orow0, wq0 + l32, nq, p.o_rs, p.o_hs, W.h, g,
+                             output_scale(p, orow0 + (wq0 + l32 < nq ? wq0 + l32 : nq - 1)));
     }
     };  // process_item
     int parity = 0;  // two hand-over words used in turn: a wave may still be reading one when thread 0, an item

@@ -52,6 +52,8 @@ class HstuFwdArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
         ("kv_splits", ctypes.c_int32),
+        ("attn_scale", ctypes.c_void_p),
+        ("attn_scale_per_row", ctypes.c_int32),
     ]
 
 
@@ -104,6 +106,7 @@ EXPORTS = (
     "hstu_hip_check_args",
     "hstu_hip_mha_fwd",
     "hstu_hip_mha_fwd_noalloc",
+    "hstu_hip_check_contract",
     "hstu_hip_mha_bwd",
     "hstu_hip_mha_bwd_workspace_bytes",
     "hstu_hip_workspace_bytes",
@@ -142,6 +145,8 @@ def lib() -> ctypes.CDLL:
         L.hstu_hip_mha_fwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
         L.hstu_hip_mha_fwd_noalloc.restype = ctypes.c_int
         L.hstu_hip_mha_fwd_noalloc.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p]
+        L.hstu_hip_check_contract.restype = ctypes.c_int
+        L.hstu_hip_check_contract.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.c_void_p, ctypes.c_void_p]
         L.hstu_hip_mha_bwd.restype = ctypes.c_int
         L.hstu_hip_mha_bwd.argtypes = [ctypes.POINTER(HstuFwdArgs), ctypes.POINTER(HstuBwdGrads), ctypes.c_void_p]
         L.hstu_hip_mha_bwd_workspace_bytes.restype = ctypes.c_size_t
@@ -216,6 +221,32 @@ def plan_for(batch, heads, dqk, dv, total_q, total_kv, max_seq_len, delta_size=0
     return cfg.value, splits.value
 
 
+def contract_checks_enabled() -> bool:
+    """``HSTU_HIP_CHECK_CONTRACT=1`` in the environment: every forward call first validates the caller contract on the
+    device and raises instead of computing (costs a small kernel and a host synchronisation; off by default)."""
+    return os.environ.get("HSTU_HIP_CHECK_CONTRACT", "0") not in ("", "0")
+
+
+_CONTRACT_BITS = (
+    (1, "seq_offsets decrease"), (2, "a sequence is longer than max_seq_len"), (4, "num_targets outside [0, length]"),
+    (8, "fewer non-target positions than contextual_seq_len"), (16, "a sequence is shorter than delta_size"),
+)
+
+
+def check_contract(a: "HstuFwdArgs", device: torch.device) -> None:
+    """Run ``hstu_hip_check_contract`` for ``a`` and raise ``ValueError`` naming what is broken (synchronises)."""
+    report = torch.empty(4, dtype=torch.int32, device=device)
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        raise_for_status(lib().hstu_hip_check_contract(ctypes.byref(a), ctypes.c_void_p(report.data_ptr()), ctypes.c_void_p(stream)))
+    bad, first, what, ends = (int(x) for x in report.cpu())
+    if bad or ends:
+        why = [text for bit, text in _CONTRACT_BITS if what & bit]
+        if ends:
+            why.append("seq_offsets[0] != 0 or seq_offsets[-1] != number of k/v rows")
+        raise ValueError(f"hstu_hip: caller contract broken by {bad} sequence(s), first at index {first}: " + "; ".join(why))
+
+
 def _dtype_code(dt: torch.dtype) -> int:
     if dt == torch.bfloat16:
         return HSTU_BF16
@@ -249,13 +280,18 @@ def mha_fwd(
     kv_splits: int = 0,
     workspace_bytes: Optional[int] = None,
     noalloc: bool = False,
+    attn_scale: Optional[torch.Tensor] = None,
+    check_contract_first: bool = False,
 ) -> None:
     """Fill ``out`` on the current stream of ``q.device``.  All tensors are device tensors.
 
     ``workspace_bytes``: scratch to hand to the library; ``None`` = as much as it asks for.  With less it skips
     the scheduling options that do not fit (the result is the same).
     ``noalloc``: go through ``hstu_hip_mha_fwd_noalloc``, which keeps its scratch in a fixed area inside the library
-    instead (no allocation here or there; calls that overlap in time on one device must not use it together)."""
+    instead (no allocation here or there; calls that overlap in time on one device must not use it together).
+    ``check_contract_first`` (or ``HSTU_HIP_CHECK_CONTRACT=1`` in the environment): validate the caller contract on the
+    device before launching and raise ``ValueError`` if it is broken.  Without it, rows of a sequence that breaks the
+    contract (longer than ``max_seq_len``, shorter than ``delta_size``, ...) may be left UNWRITTEN in ``out``."""
     a = HstuFwdArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
     a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
@@ -286,6 +322,12 @@ def mha_fwd(
     a.tile_config = tile_config
     a.sort_by_length = 1 if sort_by_length else 0
     a.kv_splits = kv_splits
+    if attn_scale is not None:
+        # fp32 on the device, 0-dim (one factor) or [total_q] (one per query row); the caller keeps it alive
+        a.attn_scale = attn_scale.data_ptr()
+        a.attn_scale_per_row = 1 if attn_scale.dim() > 0 else 0
+    if contract_checks_enabled() or check_contract_first:
+        check_contract(a, q.device)
     workspace = None
     need = lib().hstu_hip_workspace_bytes(ctypes.byref(a))
     if workspace_bytes is not None:

@@ -56,17 +56,18 @@ class _HstuMhaFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
-                min_full_attn_seq_len, sort_by_length, tile_config, kv_splits):
+                min_full_attn_seq_len, sort_by_length, tile_config, kv_splits, attn_scale):
         q, k, v = _kernel_layout(q.detach()), _kernel_layout(k.detach()), _kernel_layout(v.detach())
         out = torch.empty((v.shape[0], v.shape[1], v.shape[2]), dtype=v.dtype, device=v.device)
         if out.numel() > 0:
             hip_backend.mha_fwd(
                 q, k, v, out, seq_offsets, num_targets, max_seq_len=max_seq_len, alpha=alpha, delta_size=0,
                 max_attn_len=max_attn_len, contextual_seq_len=contextual_seq_len, min_full_attn_seq_len=min_full_attn_seq_len,
-                tile_config=tile_config, sort_by_length=sort_by_length, kv_splits=kv_splits,
+                tile_config=tile_config, sort_by_length=sort_by_length, kv_splits=kv_splits, attn_scale=attn_scale,
             )
         ctx.save_for_backward(q, k, v, seq_offsets, *([] if num_targets is None else [num_targets]))
         ctx.has_targets = num_targets is not None
+        ctx.attn_scale = attn_scale  # a constant of the call (no gradient flows into it)
         ctx.params = (max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len)
         return out
 
@@ -84,6 +85,11 @@ class _HstuMhaFunction(torch.autograd.Function):
         # rows of sequences longer than max_seq_len are outside the contract and get no gradient
         dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
         if q.numel() > 0:
+            if ctx.attn_scale is not None:
+                # out = attn_scale[row] * N * (the result with 1 / N), so the gradients are those of the plain call for
+                # dout scaled the same way
+                factor = ctx.attn_scale * float(max_seq_len)
+                dout = dout.detach().float() * (factor.view(-1, 1, 1) if factor.dim() > 0 else factor)
             dout = _kernel_layout(dout.detach().to(q.dtype))
             hip_backend.mha_bwd(
                 dout, q, k, v, dq, dk, dv, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
@@ -91,7 +97,7 @@ class _HstuMhaFunction(torch.autograd.Function):
             )
         if wide:
             dq, dk, dv = dq.float(), dk.float(), dv.float()
-        return (dq, dk, dv) + (None,) * 10
+        return (dq, dk, dv) + (None,) * 11
 
 
 def _require_device(t: torch.Tensor, name: str) -> None:
@@ -125,7 +131,14 @@ def hstu_mha(
 ) -> torch.Tensor:
     """Jagged HSTU attention forward; returns ``[L, H, Dv]``.
 
-    ``out[r] = sum_s M(r, s) * silu(alpha * q_r . k_s) / max_seq_len * v_s`` per sequence and head.
+    ``out[r] = sum_s M(r, s) * silu(alpha * q_r . k_s) / max_seq_len * v_s`` per sequence and head
+    (``attn_scale``, one factor or one per row of ``q``, takes the place of ``1 / max_seq_len``).
+
+    Caller contract, as in the reference: ``0 <= n_b <= max_seq_len``, ``0 <= num_targets[b] <= n_b``,
+    ``n_b - num_targets[b] >= contextual_seq_len``.  It is not checked by default (that would read the offsets back);
+    rows of a sequence that breaks it may come back UNINITIALISED (the output is ``torch.empty``).  Set
+    ``HSTU_HIP_CHECK_CONTRACT=1`` in the environment to have every call validated on the device first and raise
+    ``ValueError`` instead.
     """
     torch._assert(max_seq_len > 0, "max_seq_len must be larger than 0")
     torch._assert(q.dim() == 3, "q must be 3-D")
@@ -139,7 +152,14 @@ def hstu_mha(
     _require_device(v, "v")
     _require_device(seq_offsets, "seq_offsets")
     torch._assert(dropout_pr < 1e-6, "dropout for triton path not implemented")
-    assert attn_scale is None, "attn_scale not implemented"
+    if attn_scale is not None:
+        # pt_hstu_attention.py:152-165: one factor (0-dim) or one per query row, in place of 1 / max_seq_len
+        _require_device(attn_scale, "attn_scale")
+        torch._assert(attn_scale.dim() == 0 or (attn_scale.dim() == 1 and attn_scale.shape[0] == q.shape[0]),
+                      "attn_scale must be 0-dim or hold one value per row of q")
+        if torch.is_grad_enabled() and attn_scale.requires_grad:
+            raise NotImplementedError("the HIP backend has no gradient for attn_scale; detach it")
+        attn_scale = attn_scale.detach().to(torch.float32).contiguous()
     torch._assert(k.dtype == q.dtype and v.dtype == q.dtype, "q, k and v must have the same dtype")
     if num_targets is not None:
         _require_device(num_targets, "num_targets")
@@ -151,7 +171,7 @@ def hstu_mha(
             _check_forward_only(q, k, v)
         return _HstuMhaFunction.apply(
             q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len,
-            sort_by_length, tile_config, kv_splits,
+            sort_by_length, tile_config, kv_splits, attn_scale,
         )
 
     q = _kernel_layout(q.detach())
@@ -180,6 +200,7 @@ def hstu_mha(
         tile_config=tile_config,
         sort_by_length=sort_by_length,
         kv_splits=kv_splits,
+        attn_scale=attn_scale,
     )
     return out
 

@@ -93,6 +93,13 @@ typedef struct HstuFwdArgs {
                                         `workspace`; tile configs 2 and 3 only.  The result is the same up to fp32
                                         summation order.  The reference has no such option: its kernels run one
                                         block per (sequence, head, row block) in both modes */
+    const void* attn_scale;          /* NULL, or fp32 on the device: `attn_scale` of the reference
+                                        (pt_hstu_attention.py:152-165; schema flash_api_cpu.cpp:142-235): silu(.) is
+                                        multiplied by it INSTEAD of by 1 / max_seq_len.  One value for all rows
+                                        (attn_scale_per_row = 0: the reference's 0-dim tensor) or one per query row,
+                                        jagged like q ([total_q], attn_scale_per_row = 1).  Read on the device, never
+                                        on the host.  Full form only (the reference's cached form does not take it) */
+    int32_t attn_scale_per_row;
 } HstuFwdArgs;
 
 /* Library version, major*10000 + minor*100 + patch. */
@@ -116,6 +123,18 @@ int hstu_hip_check_args(const HstuFwdArgs* args);
  * delta-query (M-FALCON) forms.
  */
 int hstu_hip_mha_fwd(const HstuFwdArgs* args, void* stream);
+
+/*
+ * Opt-in check of the caller contract, on the device (the library never reads the index arrays on the host): the
+ * counterpart of the reference's debug-build checks (flash_common.cpp:529-541, HSTU_FLASH_ATTN_DEBUG_INFO).  Writes
+ * four int32 to `report` (device memory) on `stream`: the number of sequences that break the contract, the index of the
+ * first, a bit set of what is broken (1: offsets decrease, 2: longer than max_seq_len, 4: num_targets outside
+ * [0, length], 8: fewer non-target positions than contextual_seq_len, 16: shorter than delta_size), and 1 if
+ * seq_offsets[0] != 0 or seq_offsets[batch] != total_kv.  The forward pass itself never faults on such input, but rows
+ * of an offending sequence may be left unwritten (longer than max_seq_len: the rows past it; shorter than delta_size:
+ * all its rows) or masked as the formulas happen to give; the caller reads the report back when it wants to know.
+ */
+int hstu_hip_check_contract(const HstuFwdArgs* args, int32_t* report, void* stream);
 
 /*
  * The same forward pass for callers that cannot allocate device memory: code under HIP graph capture, serving loops

@@ -35,12 +35,13 @@ def silu_slope(x: torch.Tensor) -> torch.Tensor:
 def autograd_grads(
     max_seq_len: int, alpha: float, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_offsets: torch.Tensor, dout: torch.Tensor,
     num_targets: Optional[torch.Tensor] = None, max_attn_len: int = 0, contextual_seq_len: int = 0, min_full_attn_seq_len: int = 0,
-    dtype: torch.dtype = torch.float64,
+    dtype: torch.dtype = torch.float64, attn_scale: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     q, k, v = (t.detach().to(dtype).requires_grad_() for t in (q, k, v))
     out = hstu_oracle.pytorch_hstu_mha(
         max_seq_len, alpha, q, k, v, seq_offsets, num_targets=num_targets, max_attn_len=max_attn_len,
         contextual_seq_len=contextual_seq_len, min_full_attn_seq_len=min_full_attn_seq_len,
+        attn_scale=None if attn_scale is None else attn_scale.to(dtype),
     )
     out.backward(dout.to(dtype))
     return q.grad, k.grad, v.grad

@@ -259,6 +259,7 @@ def hstu_mha_per_sequence(
     compute_dtype: torch.dtype = torch.float32,
     sequences: Optional[list] = None,
     row_ranges: Optional[list] = None,
+    attn_scale: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Same mathematics as PT:129-251, one sequence at a time at its own length.
 
@@ -268,6 +269,8 @@ def hstu_mha_per_sequence(
     ``sequences`` restricts the work to those batch indices (other rows stay zero).
     ``row_ranges`` (a list of ``(r0, r1)`` in query-row indices of a sequence, clipped to its rows) restricts it
     further to those query rows; a row's result does not depend on which other rows are evaluated with it.
+    ``attn_scale`` (PT:152-165, full form only): 0-dim, or one value per query row (jagged like ``q``); it multiplies
+    ``silu`` in place of ``1 / max_seq_len``.
     """
     H = q.shape[1]
     V = v.shape[2]
@@ -293,7 +296,12 @@ def hstu_mha_per_sequence(
         for c0, c1 in chunks:
             qb = q[q0 + c0 : q0 + c1].to(compute_dtype).transpose(0, 1)  # [H, m, D]
             s = torch.matmul(qb, kb.transpose(1, 2)) * alpha
-            s = F.silu(s) / max_seq_len
+            if attn_scale is None:
+                s = F.silu(s) / max_seq_len
+            elif attn_scale.ndim == 0:
+                s = F.silu(s) * attn_scale.to(compute_dtype)
+            else:
+                s = F.silu(s) * attn_scale[q0 + c0 : q0 + c1].to(compute_dtype).view(1, -1, 1)
             m = _seq_mask_rows(
                 n,
                 rows0 + c0,

@@ -418,3 +418,27 @@ def test_backward_rejections(pkg, dev):
     empty = pkg.hstu_mha(64, 0.2, q.bfloat16()[:0].to(dev).requires_grad_(), k.bfloat16()[:0].to(dev), v.bfloat16()[:0].to(dev),
                          torch.zeros(1, dtype=torch.int64, device=dev))
     assert empty.shape == (0, 2, 32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("per_row", [False, True])
+def test_gradients_with_attn_scale(pkg, dev, per_row):
+    """hstu_mha(..., attn_scale=a).backward(): the gradients of q, k, v against autograd (fp64) through the restated
+    forward with the same attn_scale (pt_hstu_attention.py:152-165)."""
+    print("[case] backward with attn_scale, per_row", per_row, flush=True)
+    lengths = [70, 0, 33, 129]
+    q, k, v, dout, offsets = _inputs(31, lengths, 2, 32, 32, torch.bfloat16, scale=0.5)
+    N, alpha = 160, 0.2
+    tg = torch.tensor([5, 0, 33, 0])
+    a = (torch.rand(q.shape[0], generator=torch.Generator().manual_seed(9)) + 0.5) / N if per_row else torch.tensor(1.3 / N)
+    ref = G.autograd_grads(N, alpha, q, k, v, offsets, dout, num_targets=tg, max_attn_len=40, contextual_seq_len=2, attn_scale=a)
+    qd, kd, vd = (t.to(dev).requires_grad_() for t in (q, k, v))
+    out = pkg.hstu_mha(N, alpha, qd, kd, vd, offsets.to(dev), num_targets=tg.to(dev), max_attn_len=40, contextual_seq_len=2,
+                       attn_scale=a.to(dev))
+    out.backward(dout.to(dev))
+    torch.cuda.synchronize()
+    for name, got, want in zip(("dq", "dk", "dv"), (qd.grad, kd.grad, vd.grad), ref):
+        got, want = got.float().cpu(), want.float()
+        rel = float((got - want).norm() / want.norm())
+        assert rel <= 1e-2, f"{name}: relative error {rel:.3e}"
+        assert float((got - want).abs().max()) <= 2e-2 * float(want.abs().max()), name

@@ -456,6 +456,117 @@ def test_invariants_on_device(pkg, dev):
     assert torch.equal(c, a[perm.to(dev)])
 
 
+@pytest.mark.parametrize("cfg", [1, 2, 3])
+@pytest.mark.parametrize("per_row", [False, True])
+def test_attn_scale(pkg, dev, cfg, per_row):
+    """attn_scale (pt_hstu_attention.py:152-165): one factor, or one per query row, in place of 1 / max_seq_len --
+    against the oracle, and exactly N * factor times the plain result when the factor is a power of two."""
+    _announce("attn_scale", cfg, per_row)
+    lengths = [700, 0, 130, 513, 31]
+    q, k, v, offs, t = make_case(77, lengths, 3, 64, targets=[50, 0, 3, 0, 31])
+    N, alpha, kw = 1024, 0.11, dict(max_attn_len=90, contextual_seq_len=4)
+    g = torch.Generator().manual_seed(5)
+    a = (torch.rand(q.shape[0], generator=g) + 0.5) / N if per_row else torch.tensor(0.7 / N)
+    args = (N, alpha, q.to(dev), k.to(dev), v.to(dev), offs.to(dev))
+    got = pkg.hstu_mha(*args, num_targets=t.to(dev), attn_scale=a.to(dev), tile_config=cfg, **kw)
+    torch.cuda.synchronize()
+    ref = O.hstu_mha_per_sequence(N, alpha, q.float(), k.float(), v.float(), offs, num_targets=t, attn_scale=a, **kw)
+    assert_parity(got, ref, f"attn_scale cfg {cfg} per_row {per_row}")
+    plain = pkg.hstu_mha(*args, num_targets=t.to(dev), tile_config=cfg, **kw)
+    pow2 = torch.tensor(0.25) if not per_row else torch.tensor([0.5, 2.0, 0.125, 1.0])[torch.arange(q.shape[0]) % 4]
+    scaled = pkg.hstu_mha(*args, num_targets=t.to(dev), attn_scale=pow2.to(dev), tile_config=cfg, **kw)
+    torch.cuda.synchronize()
+    want = plain.float() * (pow2.to(dev) * N).view(-1, 1, 1) if per_row else plain.float() * (0.25 * N)
+    assert torch.equal(scaled.float(), want)
+    if cfg > 1:  # the sum over the runs of a kv-split takes the same factor
+        split = pkg.hstu_mha(*args, num_targets=t.to(dev), attn_scale=a.to(dev), tile_config=cfg, kv_splits=3, **kw)
+        torch.cuda.synchronize()
+        assert_parity(split, ref, "attn_scale with a kv-split")
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_mha(*args, attn_scale=a.to(dev).requires_grad_())
+
+
+def test_native_operator_with_the_references_27_arguments(pkg, dev):
+    """torch.ops.hstu.hstu_mha called exactly as the reference's forwarder calls it (ops/hstu_attention.py:70-98: 27
+    positional arguments) and as its training wrapper does (ops/cpp/cuda_hstu_attention.py), against hstu_mha of this
+    package (bit-identical: same entry point) -- forward, the (Tensor, Tensor?) form, gradients, and refusals."""
+    _announce("torch.ops.hstu.hstu_mha")
+    lengths = [300, 0, 77, 513]
+    q, k, v, offs, t = [x.to(dev) for x in make_case(5, lengths, 2, 64, targets=[20, 0, 3, 100])]
+    N, alpha = 600, 0.11
+    for offsets_dtype in (torch.int32, torch.int64):
+        o, tg = offs.to(offsets_dtype), t.to(offsets_dtype)
+        got = torch.ops.hstu.hstu_mha(
+            N, alpha, q, k, v, o, True, tg, None, 50, 0, 3, None, None, None, False, False, 0, 0, None, 0, False, None, None, None, None, 1,
+        )
+        want = pkg.hstu_mha(N, alpha, q, k, v, o, num_targets=tg, max_attn_len=50, contextual_seq_len=3)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+    out, lse = torch.ops.hstu.hstu_mha_fwd(N, alpha, q, k, v, offs, True, t, None, 50, 0, 3, None, None, None)
+    torch.cuda.synchronize()
+    assert lse is None and torch.equal(out, want)
+    a = torch.rand(q.shape[0], device=dev) / N
+    got = torch.ops.hstu.hstu_mha(N, alpha, q, k, v, offs, True, t, a, 50, 7, 3, None, None, None, True, True)
+    want = pkg.hstu_mha(N, alpha, q, k, v, offs, num_targets=t, attn_scale=a, max_attn_len=50, contextual_seq_len=3,
+                        min_full_attn_seq_len=7, sort_by_length=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    # gradients through the dispatcher's autograd registration == those of the package's autograd function
+    qa, ka, va = (x.clone().requires_grad_() for x in (q, k, v))
+    qb, kb, vb = (x.clone().requires_grad_() for x in (q, k, v))
+    g = torch.randn_like(v)
+    torch.ops.hstu.hstu_mha(N, alpha, qa, ka, va, offs, True, t, None, 50, 0, 3, None, None, None, False, False).backward(g)
+    pkg.hstu_mha(N, alpha, qb, kb, vb, offs, num_targets=t, max_attn_len=50, contextual_seq_len=3).backward(g)
+    torch.cuda.synchronize()
+    for x, y in ((qa, qb), (ka, kb), (va, vb)):
+        assert torch.equal(x.grad, y.grad)
+    # fp8 with one-element descale tensors, bf16 out
+    (qq, qs), (kq, ks), (vq, vs) = _quantize(q.float()), _quantize(k.float()), _quantize(v.float())
+    sc = [torch.tensor([x], device=dev) for x in (qs, ks, vs)]
+    got8 = torch.ops.hstu.hstu_mha(N, alpha, qq, kq, vq, offs, True, t, None, 0, 0, 0, sc[0], sc[1], sc[2], False, False)
+    want8 = pkg.hstu_mha(N, alpha, qq, kq, vq, offs, num_targets=t, q_scale=qs, k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    assert got8.dtype == torch.bfloat16 and torch.equal(got8, want8)
+    # what is not built is refused the way TORCH_CHECK refuses
+    base = (N, alpha, q, k, v, offs, True, t, None, 0, 0, 0, None, None, None, False, False)
+    for bad in (
+        base[:6] + (False,) + base[7:],                                # not causal
+        base[:5] + (None,) + base[6:],                                 # dense layout
+        base + (0, 0, offs.to(torch.int32)),                           # cross attention
+        base + (0, 0, None, 2),                                        # softmax heads
+        base + (0, 0, None, 0, True, None, None, None, None, 2),       # groups
+        (N, alpha, q.float(), k.float(), v.float()) + base[5:],        # dtype
+    ):
+        with pytest.raises(RuntimeError):
+            torch.ops.hstu.hstu_mha(*bad)
+
+
+def test_opt_in_contract_check(pkg, dev, monkeypatch):
+    """HSTU_HIP_CHECK_CONTRACT=1: a call whose index arrays break the caller contract raises instead of leaving rows
+    unwritten (the reference checks the same things in its debug build only, flash_common.cpp:529-541)."""
+    _announce("contract check")
+    q, k, v, offs, t = [x.to(dev) for x in make_case(3, [100, 40, 7], 2, 32, targets=[5, 0, 2])]
+    monkeypatch.setenv("HSTU_HIP_CHECK_CONTRACT", "1")
+    good = pkg.hstu_mha(128, 0.1, q, k, v, offs, num_targets=t, contextual_seq_len=3)
+    monkeypatch.delenv("HSTU_HIP_CHECK_CONTRACT")
+    assert torch.equal(good, pkg.hstu_mha(128, 0.1, q, k, v, offs, num_targets=t, contextual_seq_len=3))
+    monkeypatch.setenv("HSTU_HIP_CHECK_CONTRACT", "1")
+    with pytest.raises(ValueError, match="longer than max_seq_len"):
+        pkg.hstu_mha(64, 0.1, q, k, v, offs, num_targets=t)
+    with pytest.raises(ValueError, match="num_targets outside"):
+        pkg.hstu_mha(128, 0.1, q, k, v, offs, num_targets=torch.tensor([5, 41, 2], device=dev))
+    with pytest.raises(ValueError, match="first at index 2.*contextual_seq_len"):
+        pkg.hstu_mha(128, 0.1, q, k, v, offs, num_targets=t, contextual_seq_len=6)
+    with pytest.raises(ValueError, match="seq_offsets decrease"):
+        pkg.hstu_mha(128, 0.1, q, k, v, torch.tensor([0, 100, 90, 147], device=dev))
+    with pytest.raises(ValueError, match="number of k/v rows"):
+        pkg.hstu_mha(128, 0.1, q, k, v, torch.tensor([0, 100, 140, 146], device=dev))
+    dq = q[:3 * 8].contiguous()
+    with pytest.raises(ValueError, match="shorter than delta_size"):
+        pkg.delta_hstu_mha(128, 0.1, dq, k, v, offs, num_targets=torch.tensor([8, 8, 7], device=dev))
+    torch.cuda.synchronize()
+
+
 def test_cfg2_shape_subset(pkg, dev):
     """Baseline config 2 (B=256, lengths 64..1024, H=4, d=128) at full size; oracle on a subset of sequences."""
     from generative_recommenders_amd import workloads

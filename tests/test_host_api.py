@@ -238,3 +238,33 @@ def test_workload_definitions():
         wl = workloads.make_workload(name)
         assert wl.lengths.max() <= wl.max_seq_len
         assert workloads.algorithmic_bytes(wl) > 0
+
+
+def test_native_operator_schemas_are_the_references():
+    """torch.ops.hstu.hstu_mha / hstu_mha_fwd carry the schemas of ops/cpp/hstu_attention/flash_api_cpu.cpp:142-235 of
+    the reference (argument names, order, types and defaults), so that its forwarder (ops/hstu_attention.py:50-98,
+    27 positional arguments) binds."""
+    import torch
+
+    import __graft_entry__
+
+    __graft_entry__.load_package()
+    got = str(torch.ops.hstu.hstu_mha.default._schema)
+    want = (
+        "hstu::hstu_mha(SymInt max_seq_len, float alpha, Tensor q, Tensor k, Tensor v, Tensor? seq_offsets, bool causal, "
+        "Tensor? num_targets, Tensor? attn_scale, int max_attn_len, int min_full_attn_seq_len, int contextual_seq_len, "
+        "Tensor? q_descale, Tensor? k_descale, Tensor? v_descale, bool sort_by_length, bool deterministic, int sm_margin=0, "
+        "SymInt max_q_len=0, Tensor? seq_offsets_q=None, int num_softmax_heads=0, bool training=True, "
+        "Tensor? max_seq_len_tensor=None, Tensor? contextual_seq_len_tensor=None, Tensor? max_attn_len_tensor=None, "
+        "Tensor? min_full_attn_seq_len_tensor=None, int num_groups=1, bool use_bf16_dq_accum=False) -> Tensor"
+    )
+    assert got == want
+    fwd = str(torch.ops.hstu.hstu_mha_fwd.default._schema)
+    assert fwd.startswith("hstu::hstu_mha_fwd(SymInt max_seq_len, float alpha, Tensor q, Tensor k, Tensor v, Tensor? seq_offsets, bool causal, ")
+    assert fwd.endswith("int num_groups=1) -> (Tensor, Tensor?)") and "sort_by_length" not in fwd
+    # no kernel for host tensors: the dispatcher says so (there is no CPU fallback)
+    z = torch.zeros(4, 1, 32)
+    import pytest
+
+    with pytest.raises(NotImplementedError):
+        torch.ops.hstu.hstu_mha(8, 0.1, z, z, z, torch.tensor([0, 4]), True, None, None, 0, 0, 0, None, None, None, False, False)

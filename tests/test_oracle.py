@@ -187,6 +187,24 @@ def test_invariants_scale_batch_head_and_target_permutation():
     torch.testing.assert_close(c, a[perm], atol=1e-8, rtol=1e-6)
 
 
+def test_attn_scale_is_a_factor_per_query_row_in_place_of_one_over_n():
+    """PT:152-165: with attn_scale the result is attn_scale[row] * N times the plain one -- per QUERY row (a factor per
+    key would not commute with the sum over keys), for every head alike; a 0-dim tensor scales all rows."""
+    lengths, H, D, N = [19, 0, 33, 7], 2, 16, 40
+    q, k, v, offs, t = make_case(21, lengths, H, D, targets=[3, 0, 9, 1], dtype=torch.float32)
+    kw = dict(num_targets=t, max_attn_len=11, contextual_seq_len=2)
+    plain = O.pytorch_hstu_mha(N, 0.3, q, k, v, offs, **kw)
+    a = torch.rand(q.shape[0], generator=torch.Generator().manual_seed(3)) + 0.5
+    scaled = O.pytorch_hstu_mha(N, 0.3, q, k, v, offs, attn_scale=a, **kw)
+    torch.testing.assert_close(scaled, plain * (a * N).view(-1, 1, 1), atol=1e-9, rtol=1e-5)
+    one = O.pytorch_hstu_mha(N, 0.3, q, k, v, offs, attn_scale=torch.tensor(0.125), **kw)
+    torch.testing.assert_close(one, plain * (0.125 * N), atol=1e-9, rtol=1e-5)
+    per_seq = O.hstu_mha_per_sequence(N, 0.3, q, k, v, offs, attn_scale=a, row_chunk=5, **kw)
+    torch.testing.assert_close(per_seq, scaled, atol=1e-8, rtol=1e-5)
+    per_seq1 = O.hstu_mha_per_sequence(N, 0.3, q, k, v, offs, attn_scale=torch.tensor(0.125), **kw)
+    torch.testing.assert_close(per_seq1, one, atol=1e-8, rtol=1e-5)
+
+
 def test_silu_special_values():
     # one key, one query: out = silu(alpha q k) / N * v
     for x, expect in [(0.0, 0.0), (30.0, 30.0), (-30.0, -30.0 / (1 + np.exp(30.0))), (-1.2785, -0.27846)]:
