@@ -22,11 +22,21 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0}  # MI355X dense MFMA, published
 PEAK_HBM_GBS = 8000.0
 HBM_BOUND = {"cfg2", "cfg4"}  # short sequences / cached-KV streaming: priced against HBM bandwidth
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same
-# counter reads for a plain 1 GiB copy (summaries and commands under profiles/).  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"headline": 2.414e9, "cfg2": 0.827e9, "cfg3": 1.383e9, "cfg4": 0.249e9, "cfg5": 2.281e9,
-                          "kvcat": 0.173e9, "kvtail": 0.0168e9, "uqvk": 2.953e9, "layernorm": 1.074e9, "output": 5.839e9,
-                          "normmul": 2.684e9, "bwd": 6.246e9, "bwd_stored": 4.166e10}
+
+
+def measured_traffic(key):
+    """(HBM bytes of one call, the summary they come from), read from profiles/traffic.json -- written by
+    `bench.py --profile-summary` from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, each counter scaled by
+    what it reads for a plain 1 GiB copy -- or (None, None) where nothing has been measured."""
+    from generative_recommenders_amd import profile_summary
+
+    e = profile_summary.load_traffic().get(key)
+    return (e["bytes"], e["profile"]) if e else (None, None)
+
+
+def traffic_fields(key):
+    nbytes, source = measured_traffic(key)
+    return {"traffic": nbytes, "traffic_source": source}
 
 
 def run_gpu(wl, args, pkg, workloads, torch):
@@ -59,29 +69,33 @@ def run_gpu(wl, args, pkg, workloads, torch):
 
 
 def timed_steps(step, args, torch, flush):
-    """(wall ms, HIP-event ms) per step over args.steps steps; events on the stream the kernels are launched on
-    (torch's current stream).  With `flush`, every step is timed by its own pair of events and a 512 MB fill runs
-    between steps, outside the timed intervals: the workloads priced against HBM bandwidth have working sets smaller
-    than the 256 MB Infinity Cache, and back-to-back repetitions would read them from there."""
-    if not flush:
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        start.record()
-        for _ in range(args.steps):
-            step()
-        stop.record()
-        torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / args.steps, start.elapsed_time(stop) / args.steps
-    scratch = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0")
+    """(wall ms per step, timing statistics) over args.steps steps, every step between its own pair of HIP events on the
+    stream the kernels are launched on (torch's current stream).  statistics: mean (the figure the line is computed
+    from), median, 10th and 90th percentile, number of steps.  With `flush` a 512 MB fill runs between steps, outside
+    the timed intervals: the workloads priced against HBM bandwidth have working sets smaller than the 256 MB Infinity
+    Cache, and back-to-back repetitions would read them from there."""
+    scratch = torch.empty(512 << 20, dtype=torch.uint8, device="cuda:0") if flush else None
     pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
     for i, (a, b) in enumerate(pairs):
-        scratch.fill_(i & 0xFF)
+        if flush:
+            scratch.fill_(i & 0xFF)
         a.record()
         step()
         b.record()
     torch.cuda.synchronize()
-    ev_ms = sum(a.elapsed_time(b) for a, b in pairs) / args.steps
-    return ev_ms, ev_ms
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = sorted(a.elapsed_time(b) for a, b in pairs)
+    n = len(ms)
+    stats = {"mean": sum(ms) / n, "median": ms[n // 2] if n % 2 else 0.5 * (ms[n // 2 - 1] + ms[n // 2]),
+             "p10": ms[min(n - 1, int(0.1 * n))], "p90": ms[min(n - 1, int(0.9 * n))], "n": n}
+    return (stats["mean"] if flush else wall_ms), stats
+
+
+def timing_fields(stats):
+    return {"kernel_ms": round(stats["mean"], 4), "kernel_ms_median": round(stats["median"], 4), "kernel_ms_p10": round(stats["p10"], 4),
+            "kernel_ms_p90": round(stats["p90"], 4), "timed_steps": stats["n"]}
 
 
 def run_cpu_baseline(wl, torch, workloads, budget_s=20.0):
@@ -159,7 +173,8 @@ def run_jagged(name, args, pkg, torch):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    wall_ms, ev_ms = timed_steps(step, args, torch, flush=not args.no_flush)
+    wall_ms, st = timed_steps(step, args, torch, flush=not args.no_flush)
+    ev_ms = st["mean"]
     gbs = nbytes / (ev_ms * 1e-3) / 1e9
     line = {
         "metric": "K/V cache (+) delta rows per call, GB/s moved (cfg4 sizes)", "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1,
@@ -167,8 +182,8 @@ def run_jagged(name, args, pkg, torch):
         "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
         "config": {"workload": name, "batch": B, "delta_size": delta, "row_bytes": width * 2, "history_rows": int(oc[-1])},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name), "kernel": kernel,
-                     "kernel_ms": round(ev_ms, 4), "algorithmic_bytes": nbytes},
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), **traffic_fields(name), "kernel": kernel,
+                     **timing_fields(st), "algorithmic_bytes": nbytes},
     }
     if not args.no_cpu:
         torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
@@ -236,7 +251,8 @@ def run_linear(name, args, pkg, torch):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    wall_ms, ev_ms = timed_steps(step, args, torch, flush=False)
+    wall_ms, st = timed_steps(step, args, torch, flush=False)
+    ev_ms = st["mean"]
     tflops = flops / (ev_ms * 1e-3) / 1e12
     gbs = nbytes / (ev_ms * 1e-3) / 1e9
     if flops > 0:
@@ -246,10 +262,8 @@ def run_linear(name, args, pkg, torch):
     else:
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
         value, unit = round(gbs, 1), "GB/s"
-    traffic = MEASURED_TRAFFIC_BYTES.get(name)
-    if name == "uqvk" and args.uqvk_path == 1:
-        traffic = 5.549e9  # the library path: the normalised operand written, then fetched 2-3 times
-    roof.update({"traffic": traffic, "kernel": kernel, "kernel_ms": round(ev_ms, 4),
+    traffic = traffic_fields("uqvk_library" if name == "uqvk" and args.uqvk_path == 1 else name)
+    roof.update({**traffic, "kernel": kernel, **timing_fields(st),
                  "algorithmic_flops": flops, "algorithmic_bytes": nbytes, "hbm_gbs_algorithmic": round(gbs, 1)})
     line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
@@ -301,7 +315,8 @@ def run_bwd(name, args, pkg, workloads, torch, emit=True):
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    wall_ms, ev_ms = timed_steps(step, args, torch, flush=False)
+    wall_ms, st = timed_steps(step, args, torch, flush=False)
+    ev_ms = st["mean"]
     pair_flops = 2.0 * (3 * wl.dqk + 2 * wl.dv)
     flops = workloads.algorithmic_flops(wl) / (2.0 * (wl.dqk + wl.dv)) * pair_flops
     nbytes = 2.0 * wl.total_kv * wl.heads * (4 * wl.dqk + 3 * wl.dv)  # q, k, dq, dk and v, dout, dv once each
@@ -317,9 +332,9 @@ def run_bwd(name, args, pkg, workloads, torch, emit=True):
         "pct_mfma_peak": round(100.0 * tflops / PEAK_TFLOPS[wl.dtype], 2),
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_TFLOPS[wl.dtype], "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_TFLOPS[wl.dtype], 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(name + ("_stored" if stored else "")),
+                     **traffic_fields(name + ("_stored" if stored else "")),
                      "kernel": "hstu_bwd_dkdv_kernel + " + ("hstu_bwd_dq_stored_kernel" if stored else "hstu_bwd_dq_kernel"),
-                     "kernel_ms": round(ev_ms, 4),
+                     **timing_fields(st),
                      "algorithmic_flops": flops, "algorithmic_bytes": nbytes},
     }
     if not args.no_cpu and emit:
@@ -374,7 +389,24 @@ def main():
     ap.add_argument("--no-sort", action="store_true", help="do not pass sort_by_length=True to hstu_mha")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 1 GiB device copy, so that a counter run can scale FETCH_SIZE/WRITE_SIZE")
+    ap.add_argument("--profile-summary", metavar="DIR", default=None,
+                    help="no GPU work: turn the rocprofv3 csv files under DIR (kt/, fetch/, write/, optionally sq/) into a summary "
+                         "under profiles/ and record the measured HBM traffic in profiles/traffic.json")
+    ap.add_argument("--profile-out", default=None, help="--profile-summary: file to write (default profiles/<workload>.md)")
+    ap.add_argument("--profile-kernels", default="hstu", help="--profile-summary: comma-separated substrings of the kernel names that make up one call")
+    ap.add_argument("--profile-extra", default="", help="--profile-summary: the extra bench.py arguments the profiled runs were given")
+    ap.add_argument("--profile-key", default=None, help="--profile-summary: key in profiles/traffic.json (default: the workload)")
     args = ap.parse_args()
+    if args.profile_summary:
+        import __graft_entry__
+
+        __graft_entry__.load_package()
+        from generative_recommenders_amd import profile_summary
+
+        out = args.profile_out or os.path.join(ROOT, "profiles", args.workload + ".md")
+        total = profile_summary.write_summary(args.profile_summary, args.workload, out, args.profile_kernels, args.profile_extra, args.profile_key)
+        print(f"{out}: HBM traffic of one call {total / 1e9:.3f} GB")
+        return
     if args.gpus != 1:
         print("bench.py: this path is built and measured on ONE GPU; --gpus must be 1 "
               "(sequences are independent, so N GPUs would each run the same kernel on a slice)", file=sys.stderr)
@@ -410,7 +442,8 @@ def main():
     if backward:
         run_bwd(args.workload, args, pkg, workloads, torch)
         return
-    wall_ms, ev_ms = run_gpu(wl, args, pkg, workloads, torch)
+    wall_ms, st = run_gpu(wl, args, pkg, workloads, torch)
+    ev_ms = st["mean"]
     flops = workloads.algorithmic_flops(wl)
     ref_flops = workloads.reference_convention_flops(wl)
     nbytes = workloads.algorithmic_bytes(wl)
@@ -418,18 +451,18 @@ def main():
     if wl.name in HBM_BOUND:
         ach = nbytes / (ev_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
+                "frac": round(ach / PEAK_HBM_GBS, 4), **traffic_fields(wl.name)}
     else:
         peak = PEAK_TFLOPS[wl.dtype]
         roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(tflops / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl.name)}
+                "frac": round(tflops / peak, 4), **traffic_fields(wl.name)}
     cfg, splits = pkg.ops.hip_backend.plan_for(
         batch=wl.batch, heads=wl.heads, dqk=wl.dqk, dv=wl.dv, total_q=wl.batch * wl.delta_size if wl.delta_size else wl.total_kv,
         total_kv=wl.total_kv, max_seq_len=wl.max_seq_len, delta_size=wl.delta_size, tile_config=args.tile_config,
         kv_splits=args.kv_splits, sort_by_length=wl.delta_size == 0 and not args.no_sort)
     roof["kernel"] = {1: "hstu_fwd_kernel", 2: "hstu_fwd_pp_kernel<NG=2>", 3: "hstu_fwd_pp_kernel<NG=1>"}[cfg]
     roof["kv_splits"] = splits
-    roof["kernel_ms"] = round(ev_ms, 4)
+    roof.update(timing_fields(st))
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = nbytes
     line = {
@@ -464,11 +497,12 @@ def main():
         saved = (args.steps, args.warmup)
         args.steps, args.warmup = max(10, min(args.steps, 50)), 3
         try:
-            _, ms3 = run_gpu(wl3, args, pkg, workloads, torch)
+            _, st3 = run_gpu(wl3, args, pkg, workloads, torch)
+            ms3 = st3["mean"]
             exact3 = workloads.algorithmic_flops(wl3) / (ms3 * 1e-3) / 1e12
             conv3 = workloads.reference_convention_flops(wl3) / (ms3 * 1e-3) / 1e12
             line["jagged_cfg3"] = {
-                "workload": "cfg3", "kernel_ms": round(ms3, 4), "exact_tflops": round(exact3, 2),
+                "workload": "cfg3", **timing_fields(st3), "exact_tflops": round(exact3, 2),
                 "pct_mfma_peak_exact": round(100.0 * exact3 / PEAK_TFLOPS[wl3.dtype], 2),
                 "reference_convention_tflops": round(conv3, 2),
                 "pct_mfma_peak_reference_convention": round(100.0 * conv3 / PEAK_TFLOPS[wl3.dtype], 2),

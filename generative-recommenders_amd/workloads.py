@@ -152,6 +152,22 @@ def make_workload(name: str) -> Workload:
         n = rng.integers(4096, 16385, size=16)
         t = rng.integers(64, 257, size=16)
         return Workload(name, 16, 8, 128, 128, 16384, n, num_targets=t, dtype="fp8", seed=1005)
+    if name.startswith("refbench_"):
+        # the recipe of the reference's own benchmark (ops/benchmarks/hstu_attention_bench.py:65-93, 217-271): B = 512,
+        # H = 4, d = 128, lengths from generate_sparse_seq_len(sparsity 0.95) + apply_sampling(alpha 2.0), 1..20 targets
+        # per sequence, alpha = 1 / d, inputs uniform in +-0.01, q/k/v column slices of one buffer; refbench_<N> for
+        # max_seq_len N (the reference sweeps N = 256 .. 4096 by default)
+        from .common import apply_sampling, generate_sparse_seq_len
+
+        N = int(name.split("_", 1)[1])
+        with torch.random.fork_rng(devices=[]):
+            torch.manual_seed(1001)
+            lengths = generate_sparse_seq_len(size=512, max_seq_len=N, sparsity=0.95, device=torch.device("cpu"))
+            lengths = apply_sampling(lengths, 2.0, max_seq_len=N)
+            t = torch.randint(1, 21, (512,), dtype=lengths.dtype)
+            t = torch.where(t > lengths, lengths, t)
+        return Workload(name, 512, 4, 128, 128, N, lengths.numpy().astype(np.int64), num_targets=t.numpy().astype(np.int64),
+                        alpha=1.0 / 128, seed=1001, extra={"uniform": 0.01, "fused_buffer": 1.0})
     raise ValueError(f"unknown workload {name!r}")
 
 
@@ -167,18 +183,28 @@ def make_inputs(wl: Workload, device: torch.device, dtype: Optional[torch.dtype]
     """
     if dtype is None:
         dtype = {"bf16": torch.bfloat16, "fp16": torch.float16, "fp32": torch.float32, "fp8": torch.bfloat16}[wl.dtype]
-    gen = torch.Generator(device="cpu")
-    gen.manual_seed(wl.seed)
     L = wl.total_kv
+    fused_buffer = fused_buffer or bool(wl.extra.get("fused_buffer"))
+    if L * wl.heads * (2 * wl.dqk + wl.dv) > (1 << 29) and device.type != "cpu":
+        gen = torch.Generator(device=device)  # large workloads are drawn on the device
+        where = device
+    else:
+        gen, where = torch.Generator(device="cpu"), torch.device("cpu")
+    gen.manual_seed(wl.seed)
+
+    def draw(*shape):
+        if "uniform" in wl.extra:
+            a = float(wl.extra["uniform"])
+            return (torch.rand(shape, generator=gen, device=where) * (2 * a) - a).to(dtype).to(device)
+        return (torch.randn(shape, generator=gen, device=where) * 0.1).to(dtype).to(device)
+
     if fused_buffer:
-        x = (torch.randn((L, wl.heads, 2 * wl.dqk + wl.dv), generator=gen) * 0.1).to(dtype).to(device)
+        x = draw(L, wl.heads, 2 * wl.dqk + wl.dv)
         q, k, v = torch.split(x, [wl.dqk, wl.dqk, wl.dv], dim=-1)
     else:
-        q = (torch.randn((L, wl.heads, wl.dqk), generator=gen) * 0.1).to(dtype).to(device)
-        k = (torch.randn((L, wl.heads, wl.dqk), generator=gen) * 0.1).to(dtype).to(device)
-        v = (torch.randn((L, wl.heads, wl.dv), generator=gen) * 0.1).to(dtype).to(device)
+        q, k, v = draw(L, wl.heads, wl.dqk), draw(L, wl.heads, wl.dqk), draw(L, wl.heads, wl.dv)
     if wl.delta_size > 0:
-        q = (torch.randn((wl.batch * wl.delta_size, wl.heads, wl.dqk), generator=gen) * 0.1).to(dtype).to(device)
+        q = draw(wl.batch * wl.delta_size, wl.heads, wl.dqk)
     offsets = torch.zeros(wl.batch + 1, dtype=torch.int64)
     offsets[1:] = torch.from_numpy(np.cumsum(wl.lengths.astype(np.int64)))
     nt = None if wl.num_targets is None else torch.from_numpy(wl.num_targets.astype(np.int64)).to(device)

@@ -46,6 +46,13 @@ def test_headline_line_has_the_agreed_shape():
     roof = line["roofline"]
     assert roof["bound"] == "mfma" and roof["peak"] == 2500.0 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert abs(roof["achieved"] - line["value"]) < 0.1
+    # per-step HIP events: mean (what the line is computed from), median and spread, and how many steps
+    assert roof["timed_steps"] == 3 and roof["kernel_ms_p10"] <= roof["kernel_ms_median"] <= roof["kernel_ms_p90"]
+    assert roof["kernel_ms_p10"] <= roof["kernel_ms"] <= roof["kernel_ms_p90"] * 1.0001
+    # the measured HBM traffic comes from the tracked table next to the profile summaries, never from a literal here
+    table = json.load(open(os.path.join(ROOT, "profiles", "traffic.json")))
+    assert roof["traffic"] == table["headline"]["bytes"] and roof["traffic_source"] == table["headline"]["profile"]
+    assert os.path.exists(os.path.join(ROOT, roof["traffic_source"]))
     cpu = line["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["unit"] == "TFLOP/s" and cpu["sample"]
 
@@ -61,3 +68,14 @@ def test_other_workloads_print_one_line(workload, bound):
     line = _one_line(_bench("--workload", workload, "--steps", "3", "--warmup", "1", "--no-cpu"))
     assert KEYS <= set(line) and line["config"]["workload"] == workload and line["roofline"]["bound"] == bound
     assert 0.0 < line["roofline"]["frac"] < 1.0 and line["value"] > 0
+    assert {"kernel_ms", "kernel_ms_median", "kernel_ms_p10", "kernel_ms_p90", "timed_steps", "traffic", "traffic_source"} <= set(line["roofline"])
+
+
+def test_no_traffic_literal_in_bench_and_table_points_at_summaries():
+    """`roofline.traffic` is read from profiles/traffic.json, which the command that writes a summary also writes."""
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    assert "MEASURED_TRAFFIC" not in src and "traffic.json" in src
+    table = json.load(open(os.path.join(ROOT, "profiles", "traffic.json")))
+    assert "headline" in table
+    for key, entry in table.items():
+        assert entry["bytes"] > 0 and os.path.exists(os.path.join(ROOT, entry["profile"])), key
