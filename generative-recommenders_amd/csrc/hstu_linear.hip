@@ -314,14 +314,25 @@ struct GemmPlan {
     hipblasLtMatmulHeuristicResult_t candidates[kGemmCandidates];
     int ncandidates = 0;
     bool tuned = false;
+    long long rows = -1;        // what the layouts b, c, d are built for at the moment
+    long long algo_rows = -1;   // what the heuristic was asked about
 };
 
+// The number of rows (the total length of a jagged batch) changes from batch to batch, so plans are kept per size class of
+// it: the power of two below it and the two bits after that (classes a factor 1.19 .. 1.25 wide, at most 4 per octave).
+// That bounds the table by the number of distinct layer shapes times ~130, and one heuristic query serves every batch
+// of a class; the three layouts that hold the row count are rebuilt when it differs from the previous call's.
+int rows_class(long long rows) {
+    const int e = 63 - __builtin_clzll((unsigned long long)rows);
+    return e * 4 + (e >= 2 ? (int)((rows >> (e - 2)) & 3) : 0);
+}
+
 struct GemmShape {
-    long long rows, ldw, ldact, ldres, ldd;
-    int k, n, dtype, epi, device;
+    long long ldw, ldact, ldres, ldd;
+    int rows_class, k, n, dtype, epi, device;
     bool operator<(const GemmShape& o) const {
-        return std::tie(rows, ldw, ldact, ldres, ldd, k, n, dtype, epi, device) <
-               std::tie(o.rows, o.ldw, o.ldact, o.ldres, o.ldd, o.k, o.n, o.dtype, o.epi, o.device);
+        return std::tie(rows_class, ldw, ldact, ldres, ldd, k, n, dtype, epi, device) <
+               std::tie(o.rows_class, o.ldw, o.ldact, o.ldres, o.ldd, o.k, o.n, o.dtype, o.epi, o.device);
     }
 };
 
@@ -343,11 +354,42 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
     if (!g_handle && (st = hipblasLtCreate(&g_handle)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtCreate", st);
     int dev = 0;
     (void)hipGetDevice(&dev);
-    const GemmShape key{(long long)rows, (long long)ldw, (long long)ldact, (long long)ldres, (long long)ldd, k, n, dtype, epi, dev};
+    const GemmShape key{(long long)ldw, (long long)ldact, (long long)ldres, (long long)ldd, rows_class(rows), k, n, dtype, epi, dev};
+    const hipDataType t = dtype == 0 ? HIP_R_16BF : HIP_R_16F;
+    auto set_rows = [&](GemmPlan& pl) -> hipblasStatus_t {
+        if (pl.rows == rows) return HIPBLAS_STATUS_SUCCESS;
+        for (hipblasLtMatrixLayout_t* l : {&pl.b, &pl.c, &pl.d})
+            if (*l) (void)hipblasLtMatrixLayoutDestroy(*l), *l = nullptr;
+        pl.rows = -1;
+        hipblasStatus_t s;
+        if ((s = hipblasLtMatrixLayoutCreate(&pl.b, t, k, rows, ldact)) != HIPBLAS_STATUS_SUCCESS ||
+            (s = hipblasLtMatrixLayoutCreate(&pl.c, t, n, rows, residual ? ldres : ldd)) != HIPBLAS_STATUS_SUCCESS ||
+            (s = hipblasLtMatrixLayoutCreate(&pl.d, t, n, rows, ldd)) != HIPBLAS_STATUS_SUCCESS)
+            return s;
+        pl.rows = rows;
+        return HIPBLAS_STATUS_SUCCESS;
+    };
+    auto ask_heuristic = [&](GemmPlan& pl) -> hipblasStatus_t {
+        hipblasLtMatmulPreference_t pref;
+        hipblasStatus_t s;
+        if ((s = hipblasLtMatmulPreferenceCreate(&pref)) != HIPBLAS_STATUS_SUCCESS) return s;
+        const uint64_t max_ws = kGemmScratch;
+        hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
+        int found = 0;
+        s = hipblasLtMatmulAlgoGetHeuristic(g_handle, pl.desc, pl.a, pl.b, pl.c, pl.d, pref, kGemmCandidates, pl.candidates, &found);
+        hipblasLtMatmulPreferenceDestroy(pref);
+        if (s == HIPBLAS_STATUS_SUCCESS && found < 1) s = HIPBLAS_STATUS_NOT_SUPPORTED;
+        if (s != HIPBLAS_STATUS_SUCCESS) return s;
+        pl.ncandidates = found;
+        pl.algo = pl.candidates[0].algo;
+        pl.workspace = pl.candidates[0].workspaceSize;
+        pl.algo_rows = rows;
+        pl.tuned = false;
+        return s;
+    };
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
         GemmPlan pl;
-        const hipDataType t = dtype == 0 ? HIP_R_16BF : HIP_R_16F;
         if ((st = hipblasLtMatmulDescCreate(&pl.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F)) != HIPBLAS_STATUS_SUCCESS)
             return blaslt_fail("hipblasLtMatmulDescCreate", st);
         if (epi != kEpiNone) {
@@ -362,25 +404,13 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
                 st = hipblasLtMatmulDescSetAttribute(pl.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
             if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmulDescSetAttribute", st);
         }
-        if ((st = hipblasLtMatrixLayoutCreate(&pl.a, t, n, k, ldw)) != HIPBLAS_STATUS_SUCCESS ||
-            (st = hipblasLtMatrixLayoutCreate(&pl.b, t, k, rows, ldact)) != HIPBLAS_STATUS_SUCCESS ||
-            (st = hipblasLtMatrixLayoutCreate(&pl.c, t, n, rows, residual ? ldres : ldd)) != HIPBLAS_STATUS_SUCCESS ||
-            (st = hipblasLtMatrixLayoutCreate(&pl.d, t, n, rows, ldd)) != HIPBLAS_STATUS_SUCCESS)
+        if ((st = hipblasLtMatrixLayoutCreate(&pl.a, t, n, k, ldw)) != HIPBLAS_STATUS_SUCCESS || (st = set_rows(pl)) != HIPBLAS_STATUS_SUCCESS)
             return blaslt_fail("hipblasLtMatrixLayoutCreate", st);
-        hipblasLtMatmulPreference_t pref;
-        if ((st = hipblasLtMatmulPreferenceCreate(&pref)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("preference", st);
-        const uint64_t max_ws = kGemmScratch;
-        hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &max_ws, sizeof(max_ws));
-        int found = 0;
-        st = hipblasLtMatmulAlgoGetHeuristic(g_handle, pl.desc, pl.a, pl.b, pl.c, pl.d, pref, kGemmCandidates, pl.candidates, &found);
-        hipblasLtMatmulPreferenceDestroy(pref);
-        if (st != HIPBLAS_STATUS_SUCCESS || found < 1) return blaslt_fail("hipblasLtMatmulAlgoGetHeuristic", st);
-        pl.ncandidates = found;
-        pl.algo = pl.candidates[0].algo;
-        pl.workspace = pl.candidates[0].workspaceSize;
+        if ((st = ask_heuristic(pl)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmulAlgoGetHeuristic", st);
         it = g_plans.emplace(key, pl).first;
     }
     GemmPlan& pl = it->second;
+    if ((st = set_rows(pl)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatrixLayoutCreate", st);
     if (epi != kEpiNone) {
         st = hipblasLtMatmulDescSetAttribute(pl.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
         if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("bias pointer", st);
@@ -435,7 +465,13 @@ int gemm(const void* act, int64_t ldact, const void* weight, int64_t ldw, const 
         }
     }
     st = hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out, pl.d, &pl.algo,
-                         scratch, pl.workspace, stream);
+                         scratch, kGemmScratch, stream);  // all of it: the need may grow with the rows within a size class
+    if (st != HIPBLAS_STATUS_SUCCESS && pl.algo_rows != rows) {
+        // the choice made for another row count of the same size class does not take this one: ask for this one
+        if ((st = ask_heuristic(pl)) != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmulAlgoGetHeuristic", st);
+        st = hipblasLtMatmul(g_handle, pl.desc, &one, weight, pl.a, act, pl.b, &beta, residual ? residual : out, pl.c, out, pl.d,
+                             &pl.algo, scratch, kGemmScratch, stream);
+    }
     if (st != HIPBLAS_STATUS_SUCCESS) return blaslt_fail("hipblasLtMatmul", st);
     return 0;
 }

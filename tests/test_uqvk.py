@@ -179,6 +179,20 @@ def test_compute_uqvk(pkg, dev, L, d_model, H, attn, hidden, dtype, path):
 
 
 @pytest.mark.gpu
+def test_uqvk_with_a_total_length_that_changes_from_batch_to_batch(pkg, dev):
+    """The hipBLASLt path keeps one plan per size class of the row count, not per row count: lengths of one class
+    (1100, 1101, 1279), of others (640, 5000), and the first again, each against the oracle."""
+    d_model, H, attn, hidden = 192, 2, 64, 64  # no fused kernel for this d_model: layer-norm kernel + hipBLASLt
+    for L in (1100, 1101, 1279, 640, 5000, 1100, 1):
+        print(f"[case] uqvk changing rows {L}", flush=True)
+        x, nw, nb, w, b = _inputs(L, L, d_model, H, attn, hidden, torch.bfloat16)
+        got = pkg.hstu_compute_uqvk(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, H, attn, hidden, w.to(dev), b.to(dev), path=1)
+        torch.cuda.synchronize()
+        for name, g_, ref in zip("uqkv", got, U.compute_uqvk(x, nw, nb, 1e-6, H, attn, hidden, w, b)):
+            _close(g_, ref, f"{name} at {L} rows")
+
+
+@pytest.mark.gpu
 def test_uqvk_feeds_attention_in_place(pkg, dev):
     """q, k, v are column slices of the projection's output; hstu_mha reads them where they are."""
     import __graft_entry__
