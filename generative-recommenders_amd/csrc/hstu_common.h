@@ -97,6 +97,7 @@ struct FwdParams {
 // applied to the accumulator); `silu` maps one accumulator value to the P value that is rounded and
 // packed by `pack8`, leaving a constant factor to the output scale.
 struct Bf16 {
+    static constexpr bool PAIRWISE = false;
     typedef bf16x8_t vec8;
     typedef __bf16 elem;
     typedef __bf16 out_elem;
@@ -116,7 +117,29 @@ struct Bf16 {
         return r;
     }
 };
+// The second instruction of a pair writes the other half of the register the first one wrote, and reads that register
+// to do so; four independent instructions in between cover the latency of the first (the compiler does not see into
+// the asm, so nothing else would).  Operands 0-3: results, 4-7: packed fp16 pairs.
+#define HSTU_F16_PAIRS(op)                                                                                              \
+    "v_" op "_f16_e32 %0, %4\n\tv_" op "_f16_e32 %1, %5\n\tv_" op "_f16_e32 %2, %6\n\tv_" op "_f16_e32 %3, %7\n\t"      \
+    "v_" op "_f16_sdwa %0, %4 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"                            \
+    "v_" op "_f16_sdwa %1, %5 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"                            \
+    "v_" op "_f16_sdwa %2, %6 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1\n\t"                            \
+    "v_" op "_f16_sdwa %3, %7 dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:WORD_1"
+typedef __attribute__((ext_vector_type(2))) _Float16 h2_t;
+// r[j] = 1 / (1 + 2^t[j]) for four packed pairs: the transcendental instructions take one value each, the additions
+// two.  2^t beyond fp16 is inf and gives 0.
+__device__ __forceinline__ void sigmoid_f16_pairs(const h2_t (&t)[4], h2_t (&r)[4]) {
+    h2_t e[4];
+    asm(HSTU_F16_PAIRS("exp") : "=&v"(e[0]), "=&v"(e[1]), "=&v"(e[2]), "=&v"(e[3]) : "v"(t[0]), "v"(t[1]), "v"(t[2]), "v"(t[3]));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) e[j] = e[j] + (h2_t){(_Float16)1.0f, (_Float16)1.0f};
+    asm(HSTU_F16_PAIRS("rcp") : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3]) : "v"(e[0]), "v"(e[1]), "v"(e[2]), "v"(e[3]));
+}
+#undef HSTU_F16_PAIRS
+
 struct Fp16 {
+    static constexpr bool PAIRWISE = false;
     typedef f16x8_t vec8;
     typedef _Float16 elem;
     typedef _Float16 out_elem;
@@ -179,6 +202,31 @@ struct Fp8 {
         hi = __builtin_amdgcn_cvt_pk_fp8_f32(p[4], p[5], hi, false);
         hi = __builtin_amdgcn_cvt_pk_fp8_f32(p[6], p[7], hi, true);
         return (long)(((unsigned long)(unsigned)hi << 32) | (unsigned)lo);
+    }
+    // Eight scores of a tile without mask, two at a time in packed fp16 (P is kept to three mantissa bits, so fp16's
+    // eleven are plenty): t = raw * c1 in fp32, then per pair one conversion, two exp2, one packed add, two rcp, one
+    // packed multiply and one conversion to two e4m3 values that also applies the factor 16 and saturates -- 29 VALU
+    // issue cycles per score instead of 34.  The conversions run with MODE.FP16_OVFL = 1 (saturate at +-448 instead of
+    // NaN), everything in front of them with 0, so that a 2^t beyond fp16 is inf and p = t * 0 = 0 as it should be.
+    static constexpr bool PAIRWISE = true;
+    static __device__ __forceinline__ vec8 silu_pack8(const float (&raw)[8], float c1) {
+        // stage by stage over the four pairs, so that no instruction waits for the one in front of it
+        h2_t t[4], r[4], p[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t[j] = __builtin_bit_cast(h2_t, __builtin_amdgcn_cvt_pkrtz(raw[2 * j] * c1, raw[2 * j + 1] * c1));
+        sigmoid_f16_pairs(t, r);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) p[j] = t[j] * r[j];
+        // (volatile, and the mode switch inside: the compiler does not know that the conversions depend on the mode)
+        unsigned lo, hi;
+        asm volatile(
+            "s_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 1\n\ts_nop 1\n\t"
+            "v_cvt_scalef32_pk_fp8_f16 %0, %2, %6\n\tv_cvt_scalef32_pk_fp8_f16 %1, %4, %6\n\t"
+            "v_cvt_scalef32_pk_fp8_f16 %0, %3, %6 op_sel:[0,0,1]\n\tv_cvt_scalef32_pk_fp8_f16 %1, %5, %6 op_sel:[0,0,1]\n\t"
+            "s_nop 0\n\ts_setreg_imm32_b32 hwreg(HW_REG_MODE, 23, 1), 0"
+            : "=&v"(lo), "=&v"(hi)
+            : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(1.0f / PSCALE));
+        return (long)(((unsigned long)hi << 32) | lo);
     }
 };
 
@@ -598,6 +646,17 @@ struct RowMask {
 template <class TT, int MASK>
 __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (&pb)[2], float c1, const SeqMask& M,
                                           const RowMask& row, int sp0) {
+    if constexpr (MASK == 0 && TT::PAIRWISE) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            float raw[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) raw[j] = s[half * 8 + j];
+            pb[half] = TT::silu_pack8(raw, c1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+    }
     const int causal_room = row.pos - sp0;  // a key at offset d from sp0 is visible iff d <= causal_room
     unsigned bits = 0;
     if (MASK == 1) bits = row.valid_bits(sp0);
