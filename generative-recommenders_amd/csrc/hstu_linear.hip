@@ -13,6 +13,7 @@
 #include <tuple>
 
 #include "hstu_uqvk_kernel.h"
+#include "hstu_output_kernel.h"
 
 namespace {
 
@@ -243,6 +244,61 @@ __global__ __launch_bounds__(256) void hstu_norm_mul_kernel(NormMulParams p) {
 int output_blocks(const HstuOutputArgs* a) {
     if (a->group_norm) return (a->concat_u && a->concat_x) ? 3 : 1;
     return 1 + (a->concat_u ? 1 : 0) + (a->concat_x ? 1 : 0);
+}
+
+bool output_fused_shape(const HstuOutputArgs* a) {
+    const int64_t d = (int64_t)a->heads * a->linear_dim;
+    if (a->d_out != hstu::kOutCols || d < 32 || d > 1024 || (d & 31) != 0 || (a->dtype != 0 && a->dtype != 1)) return false;
+    if (a->group_norm) {
+        const int gl = a->linear_dim / 8;
+        if (a->linear_dim < 32 || (a->linear_dim & 7) != 0 || (gl & (gl - 1)) != 0 || a->heads > hstu::kOutMaxHeads) return false;
+    }
+    return true;
+}
+
+template <class TT, bool GROUP>
+int launch_output_fused_t(const hstu::OutputFusedParams& p, hipStream_t stream) {
+    auto kern = hstu::hstu_output_fused_kernel<TT, GROUP>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, hstu::kOutLds);
+        if (e != hipSuccess) {
+            snprintf(g_last_error, sizeof(g_last_error), "hipFuncSetAttribute: %s", hipGetErrorString(e));
+            return -7;
+        }
+        attr_done = true;
+    }
+    const long long grid = (p.rows + hstu::kOutRows - 1) / hstu::kOutRows;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(hstu::kOutWaves * 64), hstu::kOutLds, stream, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        snprintf(g_last_error, sizeof(g_last_error), "fused output kernel launch: %s", hipGetErrorString(e));
+        return -7;
+    }
+    return 0;
+}
+
+// The caller has checked output_fused_shape(a) and the pointers of x, output_weight, out.
+int launch_output_fused(const HstuOutputArgs* a, hipStream_t stream) {
+    const int d = a->heads * a->linear_dim;
+    if (a->attn_row_stride < d || a->u_row_stride < d) return -5;
+    if (((a->attn_row_stride | a->u_row_stride) & 7) != 0) return -4;
+    if (a->mul_u_activation < 0 || a->mul_u_activation > 2) return -5;
+    if (!a->attn || !a->u || !a->norm_weight || !a->norm_bias) return -1;
+    if ((((uintptr_t)a->attn | (uintptr_t)a->u) & 15) != 0) return -4;
+    if (!a->group_norm && (((uintptr_t)a->norm_weight | (uintptr_t)a->norm_bias) & 15) != 0) return -4;
+    const int blocks = output_blocks(a);
+    hstu::OutputFusedParams p;
+    p.attn = (const char*)a->attn, p.u = (const char*)a->u, p.x = (const char*)a->x;
+    p.attn_rs = a->attn_row_stride, p.u_rs = a->u_row_stride, p.x_rs = a->x_row_stride;
+    p.norm_weight = (const char*)a->norm_weight, p.norm_bias = (const char*)a->norm_bias, p.eps = a->norm_eps;
+    p.w = (const char*)a->output_weight, p.out = (char*)a->out, p.rows = a->rows;
+    p.d = d, p.heads = a->heads, p.group_lanes = a->group_norm ? a->linear_dim / 8 : 0;
+    p.blk_u = (blocks == 3 || (!a->group_norm && a->concat_u)) ? 1 : 0;
+    p.blk_x = (blocks == 3 || (!a->group_norm && a->concat_x)) ? 1 : 0;
+    p.silu_u = a->silu_u ? 1 : 0, p.mul_act = a->mul_u_activation;
+    if (a->dtype == 0) return a->group_norm ? launch_output_fused_t<hstu::Bf16, true>(p, stream) : launch_output_fused_t<hstu::Bf16, false>(p, stream);
+    return a->group_norm ? launch_output_fused_t<hstu::Fp16, true>(p, stream) : launch_output_fused_t<hstu::Fp16, false>(p, stream);
 }
 
 int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hipStream_t stream) {
@@ -585,6 +641,7 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
 
 size_t hstu_output_workspace_bytes(const HstuOutputArgs* a) {
     if (!a || a->rows <= 0 || a->heads <= 0 || a->linear_dim <= 0) return 0;
+    if (a->path == 2) return 0;
     return joined_bytes(a) + kGemmScratch;
 }
 
@@ -600,10 +657,18 @@ int hstu_output_forward(const HstuOutputArgs* a, void* stream_) {
     if (a->rows < 0 || a->heads <= 0 || a->linear_dim <= 0 || a->d_out <= 0 || (a->d_out & 7) != 0) return -5;
     if (a->rows > 0x7fffffffLL || a->x_row_stride < a->d_out || (a->x_row_stride & 7) != 0) return -5;
     if (a->rows == 0) return 0;
-    if (!a->x || !a->output_weight || !a->out || !a->workspace) return -1;
+    if (a->path < 0 || a->path > 2) return -5;
+    if (!a->x || !a->output_weight || !a->out) return -1;
     if ((((uintptr_t)a->x | (uintptr_t)a->output_weight | (uintptr_t)a->out) & 15) != 0) return -4;
-    if ((size_t)a->workspace_bytes < hstu_output_workspace_bytes(a) || ((uintptr_t)a->workspace & 255) != 0) return -4;
     hipStream_t stream = (hipStream_t)stream_;
+    if (a->path == 2 && !output_fused_shape(a)) {
+        snprintf(g_last_error, sizeof(g_last_error), "the fused output kernel takes d_out = 512, heads * linear_dim a multiple of 32 up "
+                 "to 1024 and, with group norm, linear_dim a power of two >= 32 and at most 8 heads");
+        return -6;
+    }
+    if (a->path == 2) return launch_output_fused(a, stream);
+    if (!a->workspace) return -1;
+    if ((size_t)a->workspace_bytes < joined_bytes(a) + kGemmScratch || ((uintptr_t)a->workspace & 255) != 0) return -4;
     const int k = output_blocks(a) * a->heads * a->linear_dim;
     void* joined = a->workspace;
     void* scratch = (char*)a->workspace + joined_bytes(a);

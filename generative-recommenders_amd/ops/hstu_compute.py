@@ -74,6 +74,7 @@ class HstuOutputArgs(ctypes.Structure):
         ("dtype", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
+        ("path", ctypes.c_int32),
     ]
 
 
@@ -290,9 +291,11 @@ def hstu_compute_output(
     group_norm: bool,
     recompute_y_in_backward: bool,
     kernel: HammerKernel = HammerKernel.HIP,
+    path: int = 0,
 ) -> torch.Tensor:
     """Returns ``x + joined @ output_weight`` of shape ``[L, d_model]``; ``recompute_y_in_backward`` concerns the
-    backward pass only and is ignored."""
+    backward pass only and is ignored.  ``path``: 0 or 1 = the norm-mul kernel + hipBLASLt (the default), 2 = the fused
+    kernel (``NotImplementedError`` if the shape does not fit; slower than the default at the benchmark's shape)."""
     _no_dropout(dropout_ratio, training)
     torch._assert(x.dim() == 2 and x.shape[0] == attn.shape[0], "x must be 2-D with attn's row count")
     _check(x, attn, u, norm_weight, norm_bias, output_weight)
@@ -303,10 +306,12 @@ def hstu_compute_output(
     out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
     a.x, a.x_row_stride = xr.data_ptr(), max(xr.stride(0), xr.shape[1])
     a.output_weight, a.out, a.d_out = w.data_ptr(), out.data_ptr(), x.shape[1]
+    a.path = int(path)
     if x.shape[0] > 0:
         need = lib().hstu_output_workspace_bytes(ctypes.byref(a))
-        workspace = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
-        a.workspace, a.workspace_bytes = (workspace.data_ptr() + 255) & ~255, need
+        if need > 0:  # the library path: `joined` and the GEMM's scratch
+            workspace = torch.empty(need + 256, dtype=torch.uint8, device=x.device)
+            a.workspace, a.workspace_bytes = (workspace.data_ptr() + 255) & ~255, need
         with torch.cuda.device(x.device):
             stream = torch.cuda.current_stream(x.device).cuda_stream
             rc = lib().hstu_output_forward(ctypes.byref(a), ctypes.c_void_p(stream))

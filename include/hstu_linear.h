@@ -73,8 +73,12 @@ int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight
  *                           joined = u | attn | y only when concat_u AND concat_x, else y alone (as the reference)
  *              silu_u     : layer norm: the copied u block goes through SiLU; group norm: u does before both uses
  *     out = x + joined @ output_weight             [rows, d_out]
- * The norm / multiply / concatenate step is one hand-written kernel (one wave per row, HBM-bound) that writes
- * `joined` in the inputs' type; the product with the residual as the GEMM's C operand runs on hipBLASLt.
+ * Two paths (see `path`).  Library path (the default, any shape): the norm / multiply / concatenate step is one
+ * hand-written kernel (one wave per row, HBM-bound) that writes `joined` in the inputs' type; the product with the
+ * residual as the GEMM's C operand runs on hipBLASLt.  Fused path (on request): one hand-written kernel in which a
+ * workgroup makes its 128 x 32 slices of `joined` in LDS, tile by tile, and multiplies them with the weight tiles
+ * streaming through LDS; attn, u, x are read and out is written once and nothing else touches HBM -- but at the
+ * benchmark's shape it takes 1.56 ms against the library path's 1.39, which is why it is not the default.
  */
 enum { HSTU_MUL_U_NONE = 0, HSTU_MUL_U_SIGMOID = 1, HSTU_MUL_U_SILU = 2 };
 
@@ -96,8 +100,13 @@ typedef struct HstuOutputArgs {
     int32_t concat_u, concat_x, group_norm, silu_u;  /* 0 / 1 */
     int32_t mul_u_activation;  /* HSTU_MUL_U_*; layer norm only */
     int32_t dtype;             /* 0 = bf16, 1 = fp16 */
-    void* workspace;           /* hstu_output_workspace_bytes() bytes, 256-byte aligned: `joined` and the GEMM's scratch */
+    void* workspace;           /* hstu_output_workspace_bytes() bytes, 256-byte aligned: `joined` and the GEMM's scratch
+                                  (library path only; may be NULL when that function returns 0) */
     int64_t workspace_bytes;
+    int32_t path;              /* 0 or 1 = library path (norm-mul kernel + hipBLASLt); 2 = fused kernel (norm, multiply,
+                                  concatenation, product and residual in one pass, `joined` never written): needs d_out
+                                  = 512, heads * linear_dim a multiple of 32 up to 1024 and, for group norm, linear_dim a
+                                  power of two >= 32 with at most 8 heads, else status -6 */
 } HstuOutputArgs;
 
 size_t hstu_output_workspace_bytes(const HstuOutputArgs* args);

@@ -177,6 +177,47 @@ def test_compute_output(pkg, dev, N, H, ld, D, cu, cx, act, group_norm, dtype):
     assert torch.equal(zero.cpu(), x)
 
 
+FUSED_CASES = [
+    # N, H, linear_dim, concat_u, concat_x, act, group_norm; d_model is 512, the width the fused kernel is built for
+    (4099, 4, 128, True, True, "none", False),
+    (1000, 4, 128, False, True, "silu", False),
+    (1000, 4, 128, True, False, "sigmoid", False),
+    (1000, 4, 128, False, False, "none", False),
+    (1000, 4, 128, True, True, "none", True),
+    (333, 8, 64, True, True, "none", True),
+    (129, 2, 32, True, True, "silu", False),
+    (1, 8, 128, True, True, "none", False),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,H,ld,cu,cx,act,group_norm", FUSED_CASES)
+def test_compute_output_fused_kernel(pkg, dev, N, H, ld, cu, cx, act, group_norm, dtype):
+    """``path=2``: norm, multiply, concatenation, product and residual in one kernel; same bar as the library path, and
+    the two paths agree with each other."""
+    D = 512
+    print(f"[case] fused output {N} {H} {ld} {cu} {cx} {act} group={group_norm} {dtype}", flush=True)
+    blocks = _blocks(cu, cx, group_norm)
+    attn, u, x, nw, nb, w = _inputs(N + H, N, H, ld, D, blocks, group_norm, dtype)
+    args = (attn.to(dev), u.to(dev), x.to(dev), nw.to(dev), nb.to(dev), 1e-6, w.to(dev), H, ld, 0.0, False, cu, cx, act, group_norm, False)
+    got = pkg.hstu_compute_output(*args, path=2)
+    lib = pkg.hstu_compute_output(*args, path=1)
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == (N, D)
+    kw = dict(concat_u=cu, concat_x=cx, mul_u_activation_type=act, group_norm=group_norm, num_heads=H, linear_dim=ld)
+    _close(got, O.compute_output(attn, u, x, nw, nb, w, 1e-6, **kw), "fused out vs fp32 oracle")
+    _close(got, lib.float().cpu(), "fused out vs library path")
+
+
+@pytest.mark.gpu
+def test_fused_output_kernel_refuses_other_widths(pkg, dev):
+    attn, u, x, nw, nb, w = _inputs(3, 100, 4, 128, 128, 3, False, torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_compute_output(attn.to(dev), u.to(dev), x.to(dev), nw.to(dev), nb.to(dev), 1e-6, w.to(dev), 4, 128, 0.0, False, True, True,
+                                "none", False, False, path=2)
+
+
 @pytest.mark.gpu
 def test_output_with_the_library_proposals_timed(pkg, dev, monkeypatch):
     """HSTU_LINEAR_TUNING=1: the first call of a new shape runs every proposal of the GEMM library; the result is the same
