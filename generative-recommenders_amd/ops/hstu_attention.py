@@ -82,8 +82,9 @@ class _HstuMhaFunction(torch.autograd.Function):
         wide = q.dtype == torch.float32
         if wide:
             q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
-        # rows of sequences longer than max_seq_len are outside the contract and get no gradient
-        dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+        # the kernels write the gradient of every row of every sequence that keeps the contract; rows past max_seq_len of
+        # a sequence that breaks it come back uninitialised, like the forward's (HSTU_HIP_CHECK_CONTRACT=1 raises instead)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         if q.numel() > 0:
             if ctx.attn_scale is not None:
                 # out = attn_scale[row] * N * (the result with 1 / N), so the gradients are those of the plain call for
