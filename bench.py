@@ -512,6 +512,22 @@ def main():
         except Exception as exc:  # noqa: BLE001  (an extra entry must not cost the line its main figure)
             line["jagged_cfg3"] = {"workload": "cfg3", "error": f"{type(exc).__name__}: {exc}"[:300]}
         args.steps, args.warmup = saved
+    if wl.name == "headline" and not args.no_jagged:
+        # the headline's own shape with unequal lengths (1024..8192, plain causal): what the same kernel does when the
+        # batch is ragged and the work goes through the work lists instead of the arithmetic deal
+        wlr = workloads.make_workload("ragged8k")
+        saved = (args.steps, args.warmup)
+        args.steps, args.warmup = max(10, min(args.steps, 50)), 3
+        try:
+            _, str_ = run_gpu(wlr, args, pkg, workloads, torch)
+            exr = workloads.algorithmic_flops(wlr) / (str_["mean"] * 1e-3) / 1e12
+            line["ragged8k"] = {
+                "workload": "ragged8k", "lengths": "64 sequences, uniform in 1024..8192, plain causal", **timing_fields(str_),
+                "exact_tflops": round(exr, 2), "pct_mfma_peak_exact": round(100.0 * exr / PEAK_TFLOPS[wlr.dtype], 2),
+            }
+        except Exception as exc:  # noqa: BLE001
+            line["ragged8k"] = {"workload": "ragged8k", "error": f"{type(exc).__name__}: {exc}"[:300]}
+        args.steps, args.warmup = saved
     if wl.name == "headline" and not args.no_bwd:
         # the backward of the same call (dq, dk, dv from dout), measured in the same run: about half a second
         saved = (args.steps, args.warmup, args.bwd_form)

@@ -115,7 +115,7 @@ def algorithmic_bytes(wl: Workload) -> float:
 
 
 def make_workload(name: str) -> Workload:
-    """The benchmark configurations by name: ``cfg1`` .. ``cfg5`` and ``headline``."""
+    """The benchmark configurations by name: ``cfg1`` .. ``cfg5``, ``headline``, ``ragged8k``, ``refbench_<N>``."""
     if name == "cfg1":
         rng = np.random.default_rng(1001)
         return Workload(name, 8, 2, 32, 32, 128, rng.integers(16, 129, size=8), dtype="fp32", seed=1001)
@@ -132,6 +132,11 @@ def make_workload(name: str) -> Workload:
         )
     if name == "headline":
         return Workload(name, 64, 4, 128, 128, 8192, np.full(64, 8192, dtype=np.int64), seed=1000)
+    if name == "ragged8k":
+        # the headline's shape with unequal lengths (uniform in 1024..8192, plain causal): same kernel, but the work goes
+        # through the ranking, the work lists and the per-XCD counters instead of the arithmetic deal of an equal-length batch
+        rng = np.random.default_rng(1006)
+        return Workload(name, 64, 4, 128, 128, 8192, rng.integers(1024, 8193, size=64).astype(np.int64), seed=1006)
     if name == "cfg4":
         rng = np.random.default_rng(1004)
         hist = rng.integers(1024, 4097, size=32)
