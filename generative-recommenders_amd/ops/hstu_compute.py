@@ -10,7 +10,8 @@ epilogue.  ``u, q, k, v`` come back as column slices of one ``[L, (2*hidden + 2*
 normalises, multiplies and writes the concatenated operand; the product, with the residual as the GEMM's C operand,
 runs on hipBLASLt.  (``csrc/hstu_linear.hip``, ``include/hstu_linear.h``.)
 
-Forward only, device tensors only, bf16 or fp16; ``kernel`` is accepted and ignored.
+Device tensors only, bf16 or fp16; ``kernel`` is accepted and ignored.  The forward runs on the kernels above; the
+gradients come from a recomputation with the framework's operators (see ``_grads_by_recomputation``).
 """
 
 import ctypes
@@ -18,6 +19,7 @@ import os
 from typing import Optional, Tuple
 
 import torch
+import torch.nn.functional as F
 
 from ..build import LINEAR_LIB_PATH
 from ..common import HammerKernel
@@ -141,10 +143,55 @@ def _check(x: torch.Tensor, *others: torch.Tensor) -> None:
     torch._assert(x.is_cuda, "x must be CUDA tensor")
     for t in others:
         torch._assert(t.is_cuda and t.dtype == x.dtype, "all tensors must be CUDA tensors of x's dtype")
-    if torch.is_grad_enabled() and any(t.requires_grad for t in (x,) + others):
-        raise NotImplementedError(
-            "the HIP backend implements the forward pass only; call it under torch.no_grad() or detach the inputs"
-        )
+
+
+def _needs_grad(*tensors: torch.Tensor) -> bool:
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+# ---- gradients of the dense steps -----------------------------------------------------------------------------------
+# The forward of every function below runs on this package's kernels.  Their gradients are NOT hand-written: the
+# backward recomputes the step with the framework's own operators (layer / group norm, addmm on hipBLASLt) in the
+# arithmetic of the reference's PyTorch backend (fp32 norm and product with u, result rounded to the input type, then the
+# product with the weight: ops/pytorch/pt_layer_norm.py:24-39, pt_hstu_linear.py:24-124, ops/hstu_compute.py:54-104) and
+# lets autograd differentiate that -- nothing but the inputs is saved, which is what the reference's recompute_* flags
+# ask for.  It is there so that a training step can run through the package.
+
+def _layer_norm_math(x, weight, bias, eps):
+    return F.layer_norm(x.float(), (x.shape[-1],), weight.float(), bias.float(), eps).to(x.dtype)
+
+
+def _uqvk_math(x, norm_weight, norm_bias, eps, u_cols, weight, bias):
+    uvqk = torch.addmm(bias, _layer_norm_math(x, norm_weight, norm_bias, eps), weight)
+    return torch.cat([F.silu(uvqk[:, :u_cols]), uvqk[:, u_cols:]], dim=1)
+
+
+def _norm_mul_math(attn, u, weight, bias, eps, silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim):
+    a32, u32, w32, b32 = attn.float(), u.float(), weight.float(), bias.float()
+    if group_norm:
+        if silu_u:
+            u32 = F.silu(u32)
+        # written out: the framework's group-norm backward on this device returned wrong weight / bias gradients for
+        # (rows, heads, linear_dim) inputs with one group per head (fp32, checked against the CPU)
+        xh = a32.view(-1, heads, linear_dim)
+        centred = xh - xh.mean(dim=-1, keepdim=True)
+        normed = centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + eps)
+        y = u32 * (normed * w32.view(1, heads, 1) + b32.view(1, heads, 1)).reshape(a32.shape)
+        parts = [u32, a32, y] if (concat_u and concat_x) else [y]
+    else:
+        gate = torch.sigmoid(u32) if act == "sigmoid" else F.silu(u32) if act == "silu" else u32
+        y = gate * F.layer_norm(a32, (a32.shape[-1],), w32, b32, eps)
+        parts = ([F.silu(u32) if silu_u else u32] if concat_u else []) + ([a32] if concat_x else []) + [y]
+    return (torch.cat(parts, dim=1) if len(parts) > 1 else parts[0]).to(attn.dtype)
+
+
+def _grads_by_recomputation(fn, tensors, d_out):
+    """d(fn(*tensors)) / d(tensor) contracted with ``d_out``, for the tensors that want a gradient (None for the others)."""
+    with torch.enable_grad():
+        leaves = [t.detach().requires_grad_(t.requires_grad) for t in tensors]
+        wanted = [t for t in leaves if t.requires_grad]
+        got = iter(torch.autograd.grad(fn(*leaves), wanted, d_out)) if wanted else iter(())
+    return tuple(next(got) if t.requires_grad else None for t in leaves)
 
 
 def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
@@ -152,6 +199,8 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
     (``ops/pytorch/pt_layer_norm.py:24-39`` of the reference)."""
     torch._assert(x.dim() == 2, "x must be 2-D")
     _check(x, weight, bias)
+    if _needs_grad(x, weight, bias):
+        return _LayerNormFunction.apply(x, weight, bias, eps)
     x = x.detach()
     if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
         x = x.contiguous()
@@ -165,6 +214,34 @@ def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: f
         )
     _raise_for_status(rc)
     return out
+
+
+class _LayerNormFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias, eps):
+        ctx.save_for_backward(x, weight, bias)
+        ctx.eps = eps
+        with torch.no_grad():
+            return layer_norm(x, weight, bias, eps)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        eps = ctx.eps
+        return _grads_by_recomputation(lambda x, w, b: _layer_norm_math(x, w, b, eps), ctx.saved_tensors, d_out) + (None,)
+
+
+class _UqvkFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, norm_weight, norm_bias, uvqk_weight, uvqk_bias, norm_eps, num_heads, attn_dim, hidden_dim, path):
+        ctx.save_for_backward(x, norm_weight, norm_bias, uvqk_weight, uvqk_bias)
+        ctx.cfg = (norm_eps, hidden_dim * num_heads)
+        return _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, path)
+
+    @staticmethod
+    def backward(ctx, d_uvqk):
+        eps, u_cols = ctx.cfg
+        fn = lambda x, nw, nb, w, b: _uqvk_math(x, nw, nb, eps, u_cols, w, b)  # noqa: E731
+        return _grads_by_recomputation(fn, ctx.saved_tensors, d_uvqk.contiguous()) + (None,) * 5
 
 
 def hstu_compute_uqvk(
@@ -188,6 +265,19 @@ def hstu_compute_uqvk(
     torch._assert(uvqk_weight.shape == (x.shape[1], n_out), "uvqk_weight must be [d_model, (2*hidden + 2*attn) * heads]")
     torch._assert(uvqk_bias.shape == (n_out,), "uvqk_bias must be [(2*hidden + 2*attn) * heads]")
     _check(x, norm_weight, norm_bias, uvqk_weight, uvqk_bias)
+    if _needs_grad(x, norm_weight, norm_bias, uvqk_weight, uvqk_bias):
+        uvqk = _UqvkFunction.apply(x, norm_weight, norm_bias, uvqk_weight, uvqk_bias, norm_eps, num_heads, attn_dim, hidden_dim, path)
+    else:
+        uvqk = _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, path)
+    u, v, q, k = torch.split(
+        uvqk, [hidden_dim * num_heads, hidden_dim * num_heads, attn_dim * num_heads, attn_dim * num_heads], dim=1
+    )
+    return u, q.view(-1, num_heads, attn_dim), k.view(-1, num_heads, attn_dim), v.view(-1, num_heads, hidden_dim)
+
+
+def _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, path) -> torch.Tensor:
+    """The ``[L, (2*hidden + 2*attn) * H]`` buffer ``u | v | q | k`` (u through SiLU) from the kernels; no autograd."""
+    n_out = (2 * hidden_dim + 2 * attn_dim) * num_heads
     x = x.detach()
     if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
         x = x.contiguous()
@@ -211,10 +301,7 @@ def hstu_compute_uqvk(
             stream = torch.cuda.current_stream(x.device).cuda_stream
             rc = lib().hstu_uqvk_forward(ctypes.byref(a), ctypes.c_void_p(stream))
         _raise_for_status(rc)
-    u, v, q, k = torch.split(
-        uvqk, [hidden_dim * num_heads, hidden_dim * num_heads, attn_dim * num_heads, attn_dim * num_heads], dim=1
-    )
-    return u, q.view(-1, num_heads, attn_dim), k.view(-1, num_heads, attn_dim), v.view(-1, num_heads, hidden_dim)
+    return uvqk
 
 
 def _rows_ok(t: torch.Tensor) -> torch.Tensor:
@@ -253,6 +340,39 @@ def _no_dropout(dropout_ratio: float, training: bool) -> None:
         raise NotImplementedError("the HIP backend implements the dropout-free forward only (training=False or dropout_ratio=0)")
 
 
+class _NormMulFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, u, weight, bias, eps, *flags):
+        ctx.save_for_backward(x, u, weight, bias)
+        ctx.cfg = (eps,) + flags
+        silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim = flags
+        with torch.no_grad():
+            return norm_mul_dropout(x, u, weight, bias, eps, 0.0, False, silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        cfg = ctx.cfg
+        fn = lambda x, u, w, b: _norm_mul_math(x, u, w, b, *cfg)  # noqa: E731
+        return _grads_by_recomputation(fn, ctx.saved_tensors, d_out.contiguous()) + (None,) * 8
+
+
+class _OutputFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, attn, u, x, norm_weight, norm_bias, output_weight, norm_eps, num_heads, linear_dim, concat_u, concat_x, act,
+                group_norm, path):
+        ctx.save_for_backward(attn, u, x, norm_weight, norm_bias, output_weight)
+        ctx.cfg = (norm_eps, False, concat_u, concat_x, act, group_norm, num_heads, linear_dim)
+        with torch.no_grad():
+            return hstu_compute_output(attn, u, x, norm_weight, norm_bias, norm_eps, output_weight, num_heads, linear_dim, 0.0, False,
+                                       concat_u, concat_x, act, group_norm, False, path=path)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        cfg = ctx.cfg
+        fn = lambda attn, u, x, nw, nb, w: torch.addmm(x, _norm_mul_math(attn, u, nw, nb, *cfg), w)  # noqa: E731
+        return _grads_by_recomputation(fn, ctx.saved_tensors, d_out.contiguous()) + (None,) * 8
+
+
 def norm_mul_dropout(
     x: torch.Tensor, u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, dropout_ratio: float, training: bool,
     silu_u: bool = False, concat_u: bool = False, concat_x: bool = False, mul_u_activation_type: str = "none",
@@ -264,6 +384,9 @@ def norm_mul_dropout(
     _check(x, u, weight, bias)
     if not group_norm:
         num_heads, linear_dim = 1, x.shape[1]
+    if _needs_grad(x, u, weight, bias):
+        return _NormMulFunction.apply(x, u, weight, bias, eps, silu_u, concat_u, concat_x, mul_u_activation_type, group_norm,
+                                      num_heads, linear_dim)
     a, keep, blocks = _output_args(x, u, weight, bias, eps, num_heads, linear_dim, concat_u, concat_x, mul_u_activation_type, group_norm, silu_u)
     joined = torch.empty((x.shape[0], blocks * x.shape[1]), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
@@ -293,12 +416,16 @@ def hstu_compute_output(
     kernel: HammerKernel = HammerKernel.HIP,
     path: int = 0,
 ) -> torch.Tensor:
-    """Returns ``x + joined @ output_weight`` of shape ``[L, d_model]``; ``recompute_y_in_backward`` concerns the
-    backward pass only and is ignored.  ``path``: 0 or 1 = the norm-mul kernel + hipBLASLt (the default), 2 = the fused
+    """Returns ``x + joined @ output_weight`` of shape ``[L, d_model]``.  The backward always recomputes ``joined``
+    (what ``recompute_y_in_backward=True`` asks for), so the flag changes nothing.  ``path``: 0 or 1 = the norm-mul kernel + hipBLASLt (the default), 2 = the fused
     kernel (``NotImplementedError`` if the shape does not fit; slower than the default at the benchmark's shape)."""
     _no_dropout(dropout_ratio, training)
     torch._assert(x.dim() == 2 and x.shape[0] == attn.shape[0], "x must be 2-D with attn's row count")
     _check(x, attn, u, norm_weight, norm_bias, output_weight)
+    if _needs_grad(x, attn, u, norm_weight, norm_bias, output_weight):
+        torch._assert(mul_u_activation_type in MUL_U_ACTIVATIONS, "mul_u_activation_type must be none, sigmoid or silu")
+        return _OutputFunction.apply(attn, u, x, norm_weight, norm_bias, output_weight, norm_eps, num_heads, linear_dim, concat_u,
+                                     concat_x, mul_u_activation_type, group_norm, path)
     a, keep, blocks = _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_dim, concat_u, concat_x,
                                    mul_u_activation_type, group_norm, False)
     torch._assert(output_weight.shape == (blocks * attn.shape[1], x.shape[1]), "output_weight must be [blocks * heads * linear_dim, d_model]")
@@ -344,7 +471,8 @@ def hstu_preprocess_and_attention(
     enable_tma: Optional[bool] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
     """``hstu_compute_uqvk`` followed by ``hstu_mha`` on the views it returns; returns ``(u, attn_output, k, v)`` with
-    ``attn_output [L, hidden * H]``.  The ``recompute_*`` flags concern the backward pass only and are ignored."""
+    ``attn_output [L, hidden * H]``.  Differentiable through its two parts; both always recompute in the backward (what
+    the ``recompute_*`` flags ask for), so the flags change nothing."""
     from .hstu_attention import hstu_mha
 
     torch._assert(max_seq_len > 0, "max_seq_len must be larger than 0")

@@ -3,8 +3,10 @@
 Mirrors ``generative_recommenders/ops/jagged_tensors.py`` of the reference (``concat_2D_jagged`` at lines 55-100,
 ``split_2D_jagged`` at lines 102-167; semantics ``ops/pytorch/pt_jagged_tensors.py:31-173``): the per-batch
 concatenation of two jagged (or dense-per-batch) 2-D tensors and its inverse -- what ``STULayer`` uses to put
-cached and new K/V rows together for ``delta_hstu_mha`` (``modules/stu.py:84-173``).  Forward only, device tensors
-only, one backend (``kernel`` is accepted and ignored).  Output sizes follow the reference's GPU backend
+cached and new K/V rows together for ``delta_hstu_mha`` (``modules/stu.py:84-173``).  Device tensors only, one backend
+(``kernel`` is accepted and ignored).  Differentiable as in the reference (``ops/triton/triton_jagged_tensors.py:
+_Concat2DJaggedFunction / _Split2DJaggedFunction``): the gradient of the concatenation is the split of the incoming
+gradient and the other way round, run by the same two kernels.  Output sizes follow the reference's GPU backend
 (``ops/triton/triton_jagged_tensors.py:546-568, 650-682``): the concatenation has
 ``values_left.shape[0] + values_right.shape[0]`` rows, which assumes the caller contract "no sequence longer than
 ``max_len_*``".
@@ -18,11 +20,49 @@ from ..common import HammerKernel, switch_to_contiguous_if_needed
 from . import hip_backend
 
 
-def _check_forward_only(*tensors: torch.Tensor) -> None:
-    if torch.is_grad_enabled() and any(t.requires_grad for t in tensors):
-        raise NotImplementedError(
-            "the HIP backend implements the forward pass only; call it under torch.no_grad() or detach the inputs"
-        )
+def _needs_grad(*tensors: torch.Tensor) -> bool:
+    return torch.is_grad_enabled() and any(t.requires_grad for t in tensors)
+
+
+def _concat_rows(left, right, offsets_left, offsets_right, batch, max_len_left, max_len_right) -> torch.Tensor:
+    left = switch_to_contiguous_if_needed(left.detach())
+    right = switch_to_contiguous_if_needed(right.detach())
+    out = torch.empty((left.shape[0] + right.shape[0], left.shape[1]), dtype=left.dtype, device=left.device)
+    if out.numel() > 0:
+        hip_backend.jagged_copy(False, left, right, out, offsets_left, offsets_right, batch, max_len_left, max_len_right)
+    return out
+
+
+def _split_rows(values, total_left, total_right, offsets_left, offsets_right, batch, max_len_left, max_len_right):
+    joined = switch_to_contiguous_if_needed(values.detach())
+    left = torch.empty((total_left, values.shape[1]), dtype=values.dtype, device=values.device)
+    right = torch.empty((total_right, values.shape[1]), dtype=values.dtype, device=values.device)
+    if values.shape[0] > 0 and values.shape[1] > 0:
+        hip_backend.jagged_copy(True, left, right, joined, offsets_left, offsets_right, batch, max_len_left, max_len_right)
+    return left, right
+
+
+class _ConcatFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, left, right, offsets_left, offsets_right, batch, max_len_left, max_len_right):
+        ctx.meta = (left.shape[0], right.shape[0], offsets_left, offsets_right, batch, max_len_left, max_len_right)
+        return _concat_rows(left, right, offsets_left, offsets_right, batch, max_len_left, max_len_right)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        d_left, d_right = _split_rows(d_out, *ctx.meta)
+        return d_left, d_right, None, None, None, None, None
+
+
+class _SplitFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, values, total_left, total_right, offsets_left, offsets_right, batch, max_len_left, max_len_right):
+        ctx.meta = (offsets_left, offsets_right, batch, max_len_left, max_len_right)
+        return _split_rows(values, total_left, total_right, offsets_left, offsets_right, batch, max_len_left, max_len_right)
+
+    @staticmethod
+    def backward(ctx, d_left, d_right):
+        return (_concat_rows(d_left, d_right, *ctx.meta),) + (None,) * 7
 
 
 def _max_len(offsets: torch.Tensor) -> int:
@@ -59,7 +99,6 @@ def concat_2D_jagged(
     )
     torch._assert(values_left.is_cuda and values_right.is_cuda, "values must be CUDA tensors")
     torch._assert(values_left.dtype == values_right.dtype, "values_left and values_right must have the same dtype")
-    _check_forward_only(values_left, values_right)
     offsets_left = _index_tensor(offsets_left, "offsets_left")
     offsets_right = _index_tensor(offsets_right, "offsets_right")
     if offsets_left is None:
@@ -76,13 +115,9 @@ def concat_2D_jagged(
         max_len_left = _max_len(offsets_left)
     if max_len_right is None:
         max_len_right = _max_len(offsets_right)
-    left = switch_to_contiguous_if_needed(values_left.detach())
-    right = switch_to_contiguous_if_needed(values_right.detach())
-    out = torch.empty((left.shape[0] + right.shape[0], left.shape[1]), dtype=left.dtype, device=left.device)
-    if out.numel() == 0:
-        return out
-    hip_backend.jagged_copy(False, left, right, out, offsets_left, offsets_right, batch, max_len_left, max_len_right)
-    return out
+    if _needs_grad(values_left, values_right):
+        return _ConcatFunction.apply(values_left, values_right, offsets_left, offsets_right, batch, max_len_left, max_len_right)
+    return _concat_rows(values_left, values_right, offsets_left, offsets_right, batch, max_len_left, max_len_right)
 
 
 def split_2D_jagged(
@@ -112,7 +147,6 @@ def split_2D_jagged(
             "offsets_left shape[0] must be equal to offsets_right shape[0]",
         )
     torch._assert(values.is_cuda, "values must be CUDA tensor")
-    _check_forward_only(values)
     offsets_left = _index_tensor(offsets_left, "offsets_left")
     offsets_right = _index_tensor(offsets_right, "offsets_right")
     total = values.shape[0]
@@ -137,12 +171,9 @@ def split_2D_jagged(
         max_len_left = _max_len(offsets_left)
     if max_len_right is None:
         max_len_right = _max_len(offsets_right)
-    joined = switch_to_contiguous_if_needed(values.detach())
-    left = torch.empty((total_left, values.shape[1]), dtype=values.dtype, device=values.device)
-    right = torch.empty((total_right, values.shape[1]), dtype=values.dtype, device=values.device)
-    if total > 0 and values.shape[1] > 0:
-        hip_backend.jagged_copy(True, left, right, joined, offsets_left, offsets_right, batch, max_len_left, max_len_right)
-    return left, right
+    if _needs_grad(values):
+        return _SplitFunction.apply(values, total_left, total_right, offsets_left, offsets_right, batch, max_len_left, max_len_right)
+    return _split_rows(values, total_left, total_right, offsets_left, offsets_right, batch, max_len_left, max_len_right)
 
 
 def write_kv_tail(full_values: torch.Tensor, full_offsets: torch.Tensor, delta_values: torch.Tensor) -> torch.Tensor:

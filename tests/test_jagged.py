@@ -214,5 +214,34 @@ def test_jagged_wrapper_rejections(pkg, dev):
         pkg.concat_2D_jagged(8, a, a[:, :4], 2, 2)
     with pytest.raises(AssertionError, match="cannot be None at the same time"):
         pkg.split_2D_jagged(8, a, max_len_left=1, max_len_right=1)
-    with pytest.raises(NotImplementedError):
-        pkg.concat_2D_jagged(8, a.clone().requires_grad_(), a, 2, 2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed,B,ma,mb,D,da,db", [(11, 4, 20, 100, 10, False, False), (12, 8, 100, 20, 30, True, False),
+                                                   (13, 5, 37, 64, 16, False, True), (14, 3, 64, 64, 128, False, False)])
+def test_hip_concat_and_split_gradients(pkg, dev, seed, B, ma, mb, D, da, db):
+    """The gradient of a row copy is the inverse row copy: checked bit for bit against the gradients autograd derives
+    for the oracle's per-batch ``torch.cat`` (the reference's test does the same with its two backends,
+    jagged_tensors_test.py:92-112)."""
+    print(f"[case] jagged gradients {seed} {B} {ma} {mb} {D} {da} {db}", flush=True)
+    va, vb, oa, ob = _case(seed, B, ma, mb, D, da, db, torch.float32)
+    kw = dict(max_len_left=ma, max_len_right=mb, offsets_left=None if da else oa.to(dev), offsets_right=None if db else ob.to(dev))
+    a_ref, b_ref = va.clone().requires_grad_(), vb.clone().requires_grad_()
+    want = J.concat_by_batch(a_ref, b_ref, oa, ob)
+    g = torch.Generator().manual_seed(seed + 100)
+    d_out = torch.randn(want.shape, generator=g)
+    want.backward(d_out)
+    a_hip, b_hip = va.to(dev).requires_grad_(), vb.to(dev).requires_grad_()
+    got = pkg.concat_2D_jagged(ma + mb, a_hip, b_hip, **kw)
+    got.backward(d_out.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(got.detach().cpu(), want.detach())
+    assert torch.equal(a_hip.grad.cpu(), a_ref.grad) and torch.equal(b_hip.grad.cpu(), b_ref.grad)
+    # and the split: its gradient is the concatenation of the two incoming gradients
+    joined = want.detach().to(dev).requires_grad_()
+    left, right = pkg.split_2D_jagged(ma + mb, joined, **kw)
+    d_left, d_right = torch.randn(va.shape, generator=g), torch.randn(vb.shape, generator=g)
+    (left * d_left.to(dev)).sum().backward(retain_graph=True)
+    (right * d_right.to(dev)).sum().backward()
+    torch.cuda.synchronize()
+    assert torch.equal(joined.grad.cpu(), J.concat_by_batch(d_left, d_right, oa, ob))

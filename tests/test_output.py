@@ -253,8 +253,6 @@ def test_output_takes_strided_views_and_rejects_what_it_cannot_do(pkg, dev):
         pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w[:-8], H, ld, 0.0, False, True, True, "none", False, False)
     with pytest.raises(AssertionError):
         pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "tanh", False, False)
-    with pytest.raises(NotImplementedError):
-        pkg.hstu_compute_output(attn.clone().requires_grad_(), u, x, nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "none", False, False)
     with pytest.raises(NotImplementedError):  # group norm over 3 chunks per head
         pkg.norm_mul_dropout(attn[:, :48], u[:, :48], nw[:2], nb[:2], 1e-6, 0.0, False, group_norm=True, num_heads=2, linear_dim=24)
     empty = pkg.hstu_compute_output(attn[:0], u[:0], x[:0], nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "none", False, False)
@@ -294,3 +292,87 @@ def test_preprocess_and_attention_then_output(pkg, dev):
     rattn = hstu_oracle.pytorch_hstu_mha(N, alpha, rq, rk, rv, offsets).reshape(L, H * Dh)
     _close(attn, rattn, "attention output")
     _close(out, O.compute_output(rattn, ru, x, ow, ob, wo, 1e-6, concat_u=True, concat_x=True, num_heads=H, linear_dim=Dh), "layer output")
+
+
+def _grad_close(got, ref, what):
+    """2e-2 for the gradients of matrices; 1e-1 for the short parameter vectors, each entry of which is a sum of ~1e4
+    signed terms that carry the bf16 roundings of the recomputation (cancellation makes the relative error of such a
+    sum several times that of its terms)."""
+    got, ref = got.float().cpu(), ref.float()
+    assert got.shape == ref.shape and torch.isfinite(got).all(), what
+    rel = float((got - ref).norm() / ref.norm())
+    bar = 2e-2 if ref.dim() > 1 else 1e-1
+    assert rel <= bar, f"{what}: relative {rel:.3e}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,H,ld,D,cu,cx,act,group_norm", [
+    (300, 4, 32, 128, True, True, "none", False), (300, 4, 32, 128, False, True, "silu", False),
+    (300, 4, 32, 128, True, False, "sigmoid", False), (300, 2, 64, 96, True, True, "none", True), (77, 2, 64, 72, False, True, "none", True),
+])
+def test_compute_output_gradients(pkg, dev, N, H, ld, D, cu, cx, act, group_norm):
+    """Forward on the kernels, gradients by recomputation: against autograd through the fp32 oracle, for every input."""
+    print(f"[case] output gradients {N} {H} {ld} {D} {cu} {cx} {act} group={group_norm}", flush=True)
+    blocks = _blocks(cu, cx, group_norm)
+    ins = _inputs(700 + N + D, N, H, ld, D, blocks, group_norm, torch.bfloat16)
+    kw = dict(concat_u=cu, concat_x=cx, mul_u_activation_type=act, group_norm=group_norm, num_heads=H, linear_dim=ld)
+    ref_in = [t.float().requires_grad_() for t in ins]
+    attn, u, x, nw, nb, w = ref_in
+    ref = O.compute_output(attn, u, x, nw, nb, w, 1e-6, **kw)
+    d_out = torch.randn(ref.shape, generator=torch.Generator().manual_seed(9))
+    ref.backward(d_out)
+    hip_in = [t.to(dev).requires_grad_() for t in ins]
+    attn_h, u_h, x_h, nw_h, nb_h, w_h = hip_in
+    out = pkg.hstu_compute_output(attn_h, u_h, x_h, nw_h, nb_h, 1e-6, w_h, H, ld, 0.0, False, cu, cx, act, group_norm, True)
+    out.backward(d_out.to(dev).to(out.dtype))
+    torch.cuda.synchronize()
+    _close(out.detach(), ref.detach(), "out")
+    for name, h, r in zip(("attn", "u", "x", "norm_weight", "norm_bias", "output_weight"), hip_in, ref_in):
+        _grad_close(h.grad, r.grad, f"d/d{name}")
+
+
+@pytest.mark.gpu
+def test_one_layer_training_step(pkg, dev):
+    """uqvk -> attention -> output, forward and backward through the package, against autograd through the three oracles
+    (the layer of modules/stu.py:286-356 of the reference): the gradient reaches x and every parameter."""
+    import numpy as np
+
+    from oracle import hstu_oracle
+
+    H, Dh, d_model, B, N = 2, 64, 128, 4, 160
+    rng = np.random.default_rng(21)
+    lengths = rng.integers(20, N + 1, size=B)
+    offsets = torch.tensor(np.concatenate([[0], np.cumsum(lengths)]), dtype=torch.int64)
+    L = int(offsets[-1])
+    g = torch.Generator().manual_seed(22)
+    dt = torch.bfloat16
+    x = torch.randn((L, d_model), generator=g).to(dt)
+    nw, nb = (1 + 0.1 * torch.randn(d_model, generator=g)).to(dt), (0.1 * torch.randn(d_model, generator=g)).to(dt)
+    wq = (torch.randn((d_model, 4 * Dh * H), generator=g) / d_model**0.5).to(dt)
+    bq = (0.1 * torch.randn(4 * Dh * H, generator=g)).to(dt)
+    ow, ob = (1 + 0.1 * torch.randn(Dh * H, generator=g)).to(dt), (0.1 * torch.randn(Dh * H, generator=g)).to(dt)
+    wo = (torch.randn((3 * Dh * H, d_model), generator=g) / (3 * Dh * H) ** 0.5).to(dt)
+    alpha = 1.0 / Dh**0.5
+    d_out = torch.randn((L, d_model), generator=g)
+    print("[case] one layer, forward and backward", flush=True)
+    params = (x, nw, nb, wq, bq, ow, ob, wo)
+    ref_in = [t.float().requires_grad_() for t in params]
+    rx, rnw, rnb, rwq, rbq, row, rob, rwo = ref_in
+    ru, rq, rk, rv = U.compute_uqvk(rx, rnw, rnb, 1e-6, H, Dh, Dh, rwq, rbq)
+    rattn = hstu_oracle.pytorch_hstu_mha(N, alpha, rq, rk, rv, offsets).reshape(L, H * Dh)
+    rout = O.compute_output(rattn, ru, rx, row, rob, rwo, 1e-6, concat_u=True, concat_x=True, num_heads=H, linear_dim=Dh)
+    rout.backward(d_out)
+    hip_in = [t.to(dev).requires_grad_() for t in params]
+    hx, hnw, hnb, hwq, hbq, how, hob, hwo = hip_in
+    u, attn, k, v = pkg.hstu_preprocess_and_attention(hx, hnw, hnb, 1e-6, H, Dh, Dh, hwq, hbq, N, offsets.to(dev), alpha, True, None, 0, 0,
+                                                      True, True, False)
+    out = pkg.hstu_compute_output(attn, u, hx, how, hob, 1e-6, hwo, H, Dh, 0.0, False, True, True, "none", False, True)
+    out.backward(d_out.to(dev).to(dt))
+    torch.cuda.synchronize()
+    _close(out.detach(), rout.detach(), "layer output")
+    names = ("x", "norm_weight", "norm_bias", "uvqk_weight", "uvqk_bias", "output_norm_weight", "output_norm_bias", "output_weight")
+    for name, h, r in zip(names, hip_in, ref_in):
+        assert h.grad is not None, name
+        got, want = h.grad.float().cpu(), r.grad
+        rel = float((got - want).norm() / want.norm())
+        assert rel <= 3e-2, f"d/d{name}: relative {rel:.3e}"

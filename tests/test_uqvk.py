@@ -235,7 +235,76 @@ def test_uqvk_wrapper_rejections(pkg, dev):
         pkg.hstu_compute_uqvk(x, nw, nb, 1e-6, 2, 8, 16, w, b)
     with pytest.raises(RuntimeError):
         pkg.hstu_compute_uqvk(x.float(), nw.float(), nb.float(), 1e-6, 2, 8, 8, w.float(), b.float())
-    with pytest.raises(NotImplementedError):
-        pkg.hstu_compute_uqvk(x.clone().requires_grad_(), nw, nb, 1e-6, 2, 8, 8, w, b)
     empty = pkg.hstu_compute_uqvk(x[:0], nw, nb, 1e-6, 2, 8, 8, w, b)
     assert empty[0].shape == (0, 16) and empty[1].shape == (0, 2, 8)
+
+
+def test_backward_math_of_the_package_is_the_oracle_s():
+    """The backward of the dense steps recomputes them with torch operators inside the package (which may not import
+    the oracle): pin those restatements against the oracle on the CPU, every flag combination of the consumer included."""
+    import __graft_entry__
+
+    __graft_entry__.load_package()
+    from generative_recommenders_amd.ops import hstu_compute as hc
+
+    from oracle import output_oracle as O
+
+    x, nw, nb, w, b = _inputs(77, 40, 64, 2, 8, 16, torch.float32)
+    want = U.compute_uqvk(x, nw, nb, 1e-6, 2, 8, 16, w, b)
+    got = hc._uqvk_math(x, nw, nb, 1e-6, 2 * 16, w, b)
+    u, v, q, k = torch.split(got, [32, 32, 16, 16], dim=1)
+    for g_, w_ in zip((u, q.reshape(-1, 2, 8), k.reshape(-1, 2, 8), v.reshape(-1, 2, 16)), want):
+        assert torch.allclose(g_, w_, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(hc._layer_norm_math(x, nw, nb, 1e-6), U.layer_norm(x, nw, nb, 1e-6), rtol=1e-6, atol=1e-6)
+    gen = torch.Generator().manual_seed(5)
+    H, ld = 2, 32
+    attn, uu = torch.randn((30, H * ld), generator=gen), torch.randn((30, H * ld), generator=gen)
+    for group in (False, True):
+        wn = torch.randn(H if group else H * ld, generator=gen)
+        bn = torch.randn(H if group else H * ld, generator=gen)
+        for cu in (False, True):
+            for cx in (False, True):
+                for act in ("none", "sigmoid", "silu"):
+                    for su in (False, True):
+                        a_ = hc._norm_mul_math(attn, uu, wn, bn, 1e-6, su, cu, cx, act, group, H, ld)
+                        b_ = O.norm_mul(attn, uu, wn, bn, 1e-6, su, cu, cx, act, group, H, ld)
+                        assert a_.shape == b_.shape and torch.allclose(a_, b_, rtol=1e-5, atol=1e-6), (group, cu, cx, act, su)
+
+
+def _grad_close(got, ref, what):
+    """2e-2 for the gradients of matrices; 1e-1 for the short parameter vectors, each entry of which is a sum of ~1e4
+    signed terms that carry the bf16 roundings of the recomputation (cancellation makes the relative error of such a
+    sum several times that of its terms)."""
+    got, ref = got.float().cpu(), ref.float()
+    assert got.shape == ref.shape and torch.isfinite(got).all(), what
+    rel = float((got - ref).norm() / ref.norm())
+    bar = 2e-2 if ref.dim() > 1 else 1e-1
+    assert rel <= bar, f"{what}: relative {rel:.3e}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L,d_model,H,attn,hidden", [(300, 128, 2, 64, 64), (77, 192, 2, 32, 64), (1000, 512, 4, 128, 128)])
+def test_uqvk_gradients(pkg, dev, L, d_model, H, attn, hidden):
+    """Forward on the kernels, gradients by recomputation: against autograd through the fp32 oracle."""
+    print(f"[case] uqvk gradients {L} {d_model} {H} {attn} {hidden}", flush=True)
+    dt = torch.bfloat16
+    x, nw, nb, w, b = _inputs(900 + L, L, d_model, H, attn, hidden, dt)
+    ref_in = [t.float().requires_grad_() for t in (x, nw, nb, w, b)]
+    ru, rq, rk, rv = U.compute_uqvk(ref_in[0], ref_in[1], ref_in[2], 1e-6, H, attn, hidden, ref_in[3], ref_in[4])
+    gen = torch.Generator().manual_seed(3)
+    du, dq, dk, dv = [torch.randn(t.shape, generator=gen) for t in (ru, rq, rk, rv)]
+    (ru * du).sum().backward(retain_graph=True)
+    ((rq * dq).sum() + (rk * dk).sum() + (rv * dv).sum()).backward()
+    hip_in = [t.to(dev).requires_grad_() for t in (x, nw, nb, w, b)]
+    u, q, k, v = pkg.hstu_compute_uqvk(hip_in[0], hip_in[1], hip_in[2], 1e-6, H, attn, hidden, hip_in[3], hip_in[4])
+    loss = (u.float() * du.to(dev)).sum() + (q.float() * dq.to(dev)).sum() + (k.float() * dk.to(dev)).sum() + (v.float() * dv.to(dev)).sum()
+    loss.backward()
+    torch.cuda.synchronize()
+    for name, h, r in zip(("x", "norm_weight", "norm_bias", "uvqk_weight", "uvqk_bias"), hip_in, ref_in):
+        _grad_close(h.grad, r.grad, f"d/d{name}")
+    # the layer norm alone
+    xl = x.to(dev).requires_grad_()
+    pkg.layer_norm(xl, nw.to(dev), nb.to(dev), 1e-6).float().pow(2).sum().backward()
+    xr = x.float().requires_grad_()
+    U.layer_norm(xr, nw.float(), nb.float(), 1e-6).pow(2).sum().backward()
+    _grad_close(xl.grad, xr.grad, "layer norm d/dx")
