@@ -314,6 +314,7 @@ struct Work {
     int n;            // sequence length (clipped to max_seq_len)
     int nq;           // query rows of this sequence (n, or delta_size)
     int m0;           // first query row of the workgroup (index into the nq rows)
+    int m1;           // one past its last query row
     int rbase;        // sequence position of query row 0 (n - delta_size in delta mode)
     int u;            // number of non-target positions
     int split;        // which run of the kv range this workgroup takes (0 when the range is not split)
@@ -339,6 +340,26 @@ __device__ __forceinline__ void kv_tile_range(const SeqMask& M, int u, int R0, i
     jt_end = (kv_hi + bn - 1) / bn;
     jt_begin = kv_lo / bn;
 }
+
+// Query rows [m0, m1) of row block `mb` (of `bm` rows) of a sequence with `nq` query rows; false if there is no such
+// block.  In the full form without a kv split the blocks are aligned to the END of the sequence, so that the partly
+// filled block is the first one -- the one with the fewest keys -- instead of the last one, which has the most: a block
+// costs its kv range however many of its rows exist, and a batch of short ragged sequences otherwise spends
+// bm / (2 n) of its steps on rows that do not exist (a quarter of them at n = 2 bm).  Otherwise (delta form, kv
+// split: there the row-block index is also the key of the partial sums) they start at row 0.
+__device__ __forceinline__ bool row_block_rows(int nq, int mb, int bm, bool end_aligned, int& m0, int& m1) {
+    if (end_aligned) {
+        const int m = (nq + bm - 1) / bm;
+        if (mb >= m) return false;
+        m1 = nq - (m - 1 - mb) * bm;
+        m0 = m1 - bm > 0 ? m1 - bm : 0;
+        return true;
+    }
+    m0 = mb * bm;
+    m1 = m0 + bm < nq ? m0 + bm : nq;
+    return m0 < nq;
+}
+__device__ __forceinline__ bool row_blocks_end_aligned(const FwdParams& p) { return p.delta == 0 && p.kv_splits <= 1; }
 
 // Decode work item `bid` (the workgroup id in a one-item-per-workgroup launch).  Workgroup ids go round-robin
 // over the 8 XCDs, so ids congruent mod 8 share an L2: all row blocks of one (sequence, head) pair stay on one
@@ -407,9 +428,8 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     n = n > p.max_seq_len ? p.max_seq_len : n;  // rows past max_seq_len do not exist for the reference either
     w.n = n;
     w.nq = p.delta > 0 ? p.delta : n;
-    w.m0 = mb * BM;
     w.rbase = p.delta > 0 ? n - p.delta : 0;
-    if (n <= 0 || w.m0 >= w.nq || w.rbase < 0) return false;
+    if (n <= 0 || w.rbase < 0 || !row_block_rows(w.nq, mb, BM, row_blocks_end_aligned(p), w.m0, w.m1)) return false;
 
     int t = 0;
     if (p.targets) t = p.targets_i64 ? (int)HSTU_CONST(int64_t, p.targets)[w.b] : HSTU_CONST(int, p.targets)[w.b];
@@ -424,9 +444,8 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     M.max_id = w.u - M.shift;
     M.idclamp = p.targets ? M.max_id : 0x7fffffff;
 
-    const int m1 = (w.m0 + BM < w.nq ? w.m0 + BM : w.nq);
     w.R0 = w.rbase + w.m0;
-    w.R1 = w.rbase + m1 - 1;
+    w.R1 = w.rbase + w.m1 - 1;
     kv_tile_range(M, w.u, w.R0, w.R1, BN, w.jt_begin, w.jt_end);
     w.nsplit = 1;
     w.block_id = (w.b * p.H + w.h) * p.num_mb + mb;
@@ -528,9 +547,8 @@ static __global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(con
                     M.idclamp = p.targets ? M.max_id : 0x7fffffff;
                 }
             }
-            const int m0 = mb * bm;
-            if (!live || m0 >= nq) continue;
-            const int m1 = m0 + bm < nq ? m0 + bm : nq;
+            int m0, m1;
+            if (!live || !row_block_rows(nq, mb, bm, row_blocks_end_aligned(p), m0, m1)) continue;
             int jb, je;
             kv_tile_range(M, u, rbase + m0, rbase + m1 - 1, bn, jb, je);
             const int tiles = je - jb;

@@ -71,7 +71,8 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     Work W;
     if (!decode_work<BM, BN>(p, W, blockIdx.x)) return;
     const SeqMask& M = W.M;
-    const int n = W.n, nq = W.nq;
+    const int n = W.n;
+    const int nq = W.m1;  // one past the last row of this item: rows from here on are never loaded or stored
 
     // rows of this wave, as sequence positions (inclusive; wR1 < wR0 if the wave has no rows)
     const int wq0 = W.m0 + wave * (QT * 32);

@@ -140,7 +140,8 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     Work W;
     if (!decode_work<BM, BN>(p, W, bid)) return;
     const SeqMask& M = W.M;
-    const int n = W.n, nq = W.nq;
+    const int n = W.n;
+    const int nq = W.m1;  // one past the last row of this item: rows from here on are never loaded or stored
 
     const int wq0 = W.m0 + wave * 32;
     const int wR0 = W.rbase + wq0;
