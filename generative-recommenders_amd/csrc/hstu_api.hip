@@ -228,7 +228,9 @@ Plan make_plan(const HstuFwdArgs* a) {
     }
     if (pl.cfg == 0) {
         if (a->delta_size == 0) {
-            pl.cfg = avg_tiles >= 3072 / kTileRows ? 2 : 3;
+            // (measured with lengths uniform in lo..hi, H = 4, d = 128: the two tie at an average of ~1150 rows, the
+            // ping-pong kernel is 3 % ahead at 1800, 6-8 % at 2048-2560, and behind by 10 % at 544)
+            pl.cfg = avg_tiles >= 1536 / kTileRows ? 2 : 3;
         } else {
             // few long histories: 256-row blocks, whose kv range is then split below so that every CU gets one
             const long long blocks256 = (long long)a->batch * a->heads * ((a->delta_size + 255) / 256);

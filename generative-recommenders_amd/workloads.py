@@ -137,6 +137,13 @@ def make_workload(name: str) -> Workload:
         # through the ranking, the work lists and the per-XCD counters instead of the arithmetic deal of an equal-length batch
         rng = np.random.default_rng(1006)
         return Workload(name, 64, 4, 128, 128, 8192, rng.integers(1024, 8193, size=64).astype(np.int64), seed=1006)
+    if name.startswith("ragged_"):
+        # ragged_<lo>_<hi>[_<B>]: the headline's shape (H = 4, d = 128, bf16, plain causal) with B (default 64) lengths
+        # uniform in lo..hi; for looking at the kernel choice between batch shapes
+        parts = [int(x) for x in name.split("_")[1:]]
+        lo, hi, batch = parts[0], parts[1], (parts[2] if len(parts) > 2 else 64)
+        rng = np.random.default_rng(1007)
+        return Workload(name, batch, 4, 128, 128, hi, rng.integers(lo, hi + 1, size=batch).astype(np.int64), seed=1007)
     if name == "cfg4":
         rng = np.random.default_rng(1004)
         hist = rng.integers(1024, 4097, size=32)
