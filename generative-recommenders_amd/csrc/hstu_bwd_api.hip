@@ -8,6 +8,7 @@
 #include <cstring>
 
 #include "hstu_bwd_kernel.h"
+#include "hstu_bwd_pp_kernel.h"
 
 // defined with the forward entry points (hstu_api.hip); internal to the library
 extern "C" __attribute__((visibility("hidden"))) int hstu_hip_device_is_gfx950(void);
@@ -28,11 +29,28 @@ size_t ds_bytes(const HstuFwdArgs* a) {
     return ((size_t)a->total_q + 32 * (size_t)a->batch) * (size_t)a->heads * pitch32 * 64;
 }
 
+template <class TT, int DQK, int DV, bool STORE>
+auto key_stationary_kernel(std::true_type) {
+    return hstu::hstu_bwd_dkdv_pp_kernel<TT, DQK, DV, STORE>;
+}
+template <class TT, int DQK, int DV, bool STORE>
+auto key_stationary_kernel(std::false_type) {
+    return hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile, STORE>;
+}
+
 template <class TT, int DQK, int DV>
 int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
     // three tile slots for the key-stationary kernel, two for the other; + 64: transposing reads of a 16-wide tile's unused half
-    constexpr int smem1 = 3 * kBwdTile * (DQK + DV) * 2 + 64, smem = 2 * kBwdTile * (DQK + DV) * 2 + 64;
+    constexpr int smem1 = 3 * kBwdTile * (DQK + DV) * 2 + 64;
+    constexpr int smem = 2 * kBwdTile * (DQK + DV) * 2 + 64;
     constexpr int smem3 = 3 * kBwdTile * DQK * 2 + kStoredWaves * 3 * 4096;
+    // The key-stationary kernel: with two waves per SIMD where a tile copy gives every copying wave something to do and
+    // the byte offsets inside a tile of 64 rows fit its 32-bit arithmetic; the one-wave kernel otherwise.
+    constexpr bool kPairedDims = DQK >= 32 && DV >= 32;
+    auto k1p = key_stationary_kernel<TT, DQK, DV, false>(std::integral_constant<bool, kPairedDims>{});
+    auto k1ps = key_stationary_kernel<TT, DQK, DV, true>(std::integral_constant<bool, kPairedDims>{});
+    constexpr int smem1p = kPairedDims ? hstu::bwd_pp_lds_bytes<(DQK < 32 ? 32 : DQK), (DV < 32 ? 32 : DV)>() : 0;
+    const bool paired = kPairedDims && bp.f.q_rs < (1 << 22) && bp.do_rs < (1 << 22);
     auto k1 = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile, false>;
     auto k1s = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile, true>;
     auto k2 = hstu::hstu_bwd_dq_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
@@ -41,6 +59,10 @@ int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1s, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
+        if (kPairedDims) {
+            if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1p, hipFuncAttributeMaxDynamicSharedMemorySize, smem1p);
+            if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1ps, hipFuncAttributeMaxDynamicSharedMemorySize, smem1p);
+        }
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k2, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k3, hipFuncAttributeMaxDynamicSharedMemorySize, smem3);
         if (e != hipSuccess) {
@@ -51,13 +73,15 @@ int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
     }
     const unsigned grid = (unsigned)bp.f.slots_per_xcd * 8;
     if (bp.ds) {
-        hipLaunchKernelGGL(k1s, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
+        if (paired) hipLaunchKernelGGL(k1ps, dim3(grid), dim3(hstu::kBwdPpWaves * 64), smem1p, stream, bp);
+        else hipLaunchKernelGGL(k1s, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
         hstu::BwdParams b3 = bp;  // the same items in blocks of 256 query rows
         b3.f.num_mb = (bp.f.max_seq_len + kStoredRows - 1) / kStoredRows;
         b3.f.slots_per_xcd = bp.f.pairs_per_xcd * b3.f.num_mb;
         hipLaunchKernelGGL(k3, dim3((unsigned)b3.f.slots_per_xcd * 8), dim3(kStoredWaves * 64), smem3, stream, b3);
     } else {
-        hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
+        if (paired) hipLaunchKernelGGL(k1p, dim3(grid), dim3(hstu::kBwdPpWaves * 64), smem1p, stream, bp);
+        else hipLaunchKernelGGL(k1, dim3(grid), dim3(kBwdWaves * 64), smem1, stream, bp);
         hipLaunchKernelGGL(k2, dim3(grid), dim3(kBwdWaves * 64), smem, stream, bp);
     }
     hipError_t e = hipGetLastError();

@@ -59,6 +59,7 @@ __device__ __forceinline__ char* ds_pair_base(const BwdParams& bp, const Work& W
     return bp.ds + row_units * 64 + (int64_t)W.h * nqb * bp.ds_pitch32 * 2048;
 }
 
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
 constexpr int kKeyBlock = 128, kQueryTile = 64;  // geometry of the key-stationary kernel
 
 // The tiles of 64 query rows that the key-stationary kernel visits for the 128 keys starting at S0: rows at or after
@@ -217,6 +218,24 @@ __device__ __forceinline__ void silu_and_slope(float t, float& p, float& g) {
     const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t));
     p = t * sig;
     g = __builtin_fmaf(0.6931471805599453f * p, sig - 1.0f, sig);
+}
+
+// The same in two pieces whose instructions stay where they are written (the compiler does not look into the asm, so
+// the wait state between a transcendental instruction and the first ordinary one that reads its result is spelled out
+// where no other instruction stands between them).
+__device__ __forceinline__ float sigma_pinned(float t) {
+    float s;
+    asm volatile("v_exp_f32 %0, %1\n\ts_nop 0\n\tv_add_f32 %0, 1.0, %0\n\tv_rcp_f32 %0, %0" : "=v"(s) : "v"(t));
+    return s;
+}
+// p = t * sigma;  dS = dp * (sigma + p * (ln2 * sigma - ln2)).  WAIT: nothing was issued since sigma_pinned.
+template <bool WAIT>
+__device__ __forceinline__ void silu_and_slope_pinned(float t, float dp, float sig, float& p, float& ds) {
+    const float ln2 = 0.6931471805599453f;
+    if (WAIT) asm volatile("s_nop 0");
+    asm volatile("v_mul_f32 %0, %2, %3\n\tv_fma_f32 %1, %5, %3, -%5\n\tv_fma_f32 %1, %0, %1, %3\n\tv_mul_f32 %1, %4, %1"
+                 : "=&v"(p), "=&v"(ds)
+                 : "v"(t), "v"(sig), "v"(dp), "s"(ln2));
 }
 
 // ---- key-stationary kernel: dK, dV ---------------------------------------------------------------------------------
@@ -414,8 +433,12 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
         for (int k = 0; k < PD && k < NA; ++k) fa[k] = load_a(k);
 #pragma unroll
         for (int k = 0; k < PD && k < NB; ++k) fb[k] = load_b(k);
-        float pv[16], dsv[16];
-        auto mat = [&](int e) __attribute__((always_inline)) {
+        // Slot e: one product of stream A, the first half of the pointwise work on element e (sigma), one product of
+        // stream B with the copies and stores, the second half (p, the slope, dS, rounding).  A wave's VALU
+        // instructions run in the shadow of its own MFMA only when few of them follow each MFMA (up to six measured:
+        // 45 cycles per MFMA with six behind each one, 62 with twelve behind each pair), so the pointwise work is cut
+        // into pieces of four and pinned between the products.
+        auto mat_a = [&](int e) __attribute__((always_inline)) {
 #pragma unroll
             for (int k = 0; k < NA; ++k) {
                 if (k * 16 / NA != e) continue;
@@ -423,6 +446,8 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
                 else dp_n = TT::mfma(fa[k % PD], vreg[OpsA::index(k)], dp_n);
                 if (k + PD < NA) fa[k % PD] = load_a(k + PD);
             }
+        };
+        auto mat_b = [&](int e) __attribute__((always_inline)) {
 #pragma unroll
             for (int k = 0; k < NB; ++k) {
                 if (k * 16 / NB != e) continue;
@@ -450,34 +475,36 @@ __global__ __launch_bounds__(NW * 64, 1) void hstu_bwd_dkdv_kernel(const BwdPara
                 if (e == 2) *(vec8*)(dst + 1024 + (((2 * l32 + g) * 16) ^ 128) - (2 * l32 + g) * 16) = dsb_i[1];
             }
         };
-        auto pw = [&](int e) __attribute__((always_inline)) {
-            float pr, gr;
-            silu_and_slope(s_c[e], pr, gr);
-            pv[e] = pr;
-            dsv[e] = dp_c[e] * gr;
+        float sg, pe[2], de[2];
+        unsigned pk[4], dk[4];
+        auto pw_a = [&](int e) __attribute__((always_inline)) { sg = sigma_pinned(s_c[e]); };
+        auto pw_b = [&](int e) __attribute__((always_inline)) {
+            silu_and_slope_pinned<(NB < 16)>(s_c[e], dp_c[e], sg, pe[e & 1], de[e & 1]);
+            if (e & 1) {
+                pk[(e >> 1) & 3] = TT::pack2_pinned(pe[0], pe[1]);
+                dk[(e >> 1) & 3] = TT::pack2_pinned(de[0], de[1]);
+            }
             if (e == 7 || e == 15) {
-                float p8[8], d8[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    p8[j] = pv[e - 7 + j];
-                    d8[j] = dsv[e - 7 + j];
-                }
-                pb_o[e >> 3] = TT::pack8(p8);
-                dsb_o[e >> 3] = TT::pack8(d8);
+                pb_o[e >> 3] = __builtin_bit_cast(vec8, (u32x4_t){pk[0], pk[1], pk[2], pk[3]});
+                dsb_o[e >> 3] = __builtin_bit_cast(vec8, (u32x4_t){dk[0], dk[1], dk[2], dk[3]});
             }
         };
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             __builtin_amdgcn_sched_barrier(0);
-            mat(e);
-            pw(e);
+            mat_a(e);
+            __builtin_amdgcn_sched_barrier(0);
+            pw_a(e);
+            __builtin_amdgcn_sched_barrier(0);
+            mat_b(e);
+            __builtin_amdgcn_sched_barrier(0);
+            pw_b(e);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
     // Clear the entries of a packed block (first query row r0) that the mask removes: everything for class 0, the
     // pairs the predicate rejects for class 1.  Works on the rounded values, so whatever the pointwise step made of
     // rows that do not exist (even a NaN) goes away.
-    typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
     auto apply_mask = [&](int cls, int r0, vec8 (&pb_o)[2], vec8 (&dsb_o)[2]) __attribute__((always_inline)) {
         if (cls == 2) return;
         const unsigned rows = cls == 1 ? key.valid_bits(r0 + 4 * g, n) : 0u;  // bit d: row r0 + 4 g + d sees the lane's key

@@ -116,6 +116,12 @@ struct Bf16 {
         for (int j = 0; j < 8; ++j) r[j] = (elem)p[j];
         return r;
     }
+    // two values rounded as pack8 rounds them, by an instruction that stays where it is written
+    static __device__ __forceinline__ unsigned pack2_pinned(float a, float b) {
+        unsigned r;
+        asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+        return r;
+    }
 };
 // The second instruction of a pair writes the other half of the register the first one wrote, and reads that register
 // to do so; four independent instructions in between cover the latency of the first (the compiler does not see into
@@ -155,6 +161,11 @@ struct Fp16 {
         vec8 r;
 #pragma unroll
         for (int j = 0; j < 8; ++j) r[j] = (elem)p[j];
+        return r;
+    }
+    static __device__ __forceinline__ unsigned pack2_pinned(float a, float b) {
+        unsigned r, t;
+        asm volatile("v_cvt_f16_f32 %0, %2\n\tv_cvt_f16_f32 %1, %3\n\tv_pack_b32_f16 %0, %0, %1" : "=&v"(r), "=&v"(t) : "v"(a), "v"(b));
         return r;
     }
 };
