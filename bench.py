@@ -333,7 +333,7 @@ def run_bwd(name, args, pkg, workloads, torch, emit=True):
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": PEAK_TFLOPS[wl.dtype], "unit": "TFLOP/s",
                      "frac": round(tflops / PEAK_TFLOPS[wl.dtype], 4),
                      **traffic_fields(name + ("_stored" if stored else "")),
-                     "kernel": "hstu_bwd_dkdv_kernel + " + ("hstu_bwd_dq_stored_kernel" if stored else "hstu_bwd_dq_kernel"),
+                     "kernel": ("hstu_bwd_dkdv_pp_kernel" if min(wl.dqk, wl.dv) >= 32 else "hstu_bwd_dkdv_kernel") + " + " + ("hstu_bwd_dq_stored_kernel" if stored else "hstu_bwd_dq_kernel"),
                      **timing_fields(st),
                      "algorithmic_flops": flops, "algorithmic_bytes": nbytes},
     }
