@@ -169,6 +169,8 @@ GRID = [
     # B, N, H, dqk, dv, mask index
     (4, 200, 2, 64, 64, 0), (3, 300, 1, 128, 128, 0), (5, 130, 2, 32, 32, 1), (4, 257, 2, 128, 128, 4), (3, 200, 4, 64, 128, 3),
     (2, 150, 2, 16, 16, 0), (3, 180, 1, 128, 32, 5), (4, 100, 3, 16, 64, 2), (2, 520, 2, 128, 128, 1), (6, 64, 2, 32, 128, 4),
+    # longer walks of the key-stationary kernel: the tile slots wrap several times, windows end inside the walk
+    (2, 900, 2, 128, 128, 5), (2, 1100, 1, 64, 32, 4), (3, 700, 2, 32, 64, 1), (2, 1300, 1, 128, 64, 2),
 ]
 
 
