@@ -238,10 +238,11 @@ def run_linear(name, args, pkg, torch):
         nw, nb = rnd(H * D, scale=0.1, shift=1.0), rnd(H * D, scale=0.1)
         w = rnd(3 * H * D, d_model, scale=1.0 / (3 * H * D) ** 0.5)
         if name == "output":
-            step = lambda: hstu_compute.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, D, 0.0, False, True, True, "none", False, False)  # noqa: E731
+            step = lambda: hstu_compute.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, D, 0.0, False, True, True, "none", False, False, path=args.output_path)  # noqa: E731
             cpu = lambda r: output_oracle.compute_output(attn[:r].float().cpu(), u[:r].float().cpu(), x[:r].float().cpu(), nw.float().cpu(), nb.float().cpu(), w.float().cpu(), 1e-6, concat_u=True, concat_x=True)  # noqa: E731
             flops, nbytes = 2.0 * L * 3 * H * D * d_model, 2.0 * (2 * L * H * D + 2 * L * d_model + 3 * H * D * d_model)
-            kernel = "hstu_norm_mul_kernel + hipBLASLt GEMM (residual as C operand)"
+            kernel = ("hstu_norm_mul_kernel + hipBLASLt GEMM (residual as C operand)" if args.output_path == 1
+                      else "hstu_norm_mul_kernel (y alone) + hstu_output_gemm_kernel")
             metric = "hstu_compute_output fwd TFLOP/s (524288 tokens, 3 x 512 -> 512)"
         else:
             step = lambda: hstu_compute.norm_mul_dropout(attn, u, nw, nb, 1e-6, 0.0, False, False, True, True, "none")  # noqa: E731
@@ -262,7 +263,7 @@ def run_linear(name, args, pkg, torch):
     else:
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
         value, unit = round(gbs, 1), "GB/s"
-    traffic = traffic_fields("uqvk_library" if name == "uqvk" and args.uqvk_path == 1 else name)
+    traffic = traffic_fields(name + "_library" if (name == "uqvk" and args.uqvk_path == 1) or (name == "output" and args.output_path == 1) else name)
     roof.update({**traffic, "kernel": kernel, **timing_fields(st),
                  "algorithmic_flops": flops, "algorithmic_bytes": nbytes, "hbm_gbs_algorithmic": round(gbs, 1)})
     line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -374,6 +375,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="headline")
     ap.add_argument("--tile-config", type=int, default=0)
+    ap.add_argument("--output-path", type=int, default=0, help="workload output: 0 / 2 = norm-multiply kernel + concatenating GEMM kernel, 1 = norm-multiply kernel + hipBLASLt")
     ap.add_argument("--uqvk-path", type=int, default=0, help="workload uqvk: 0 / 2 = fused kernel, 1 = layer-norm kernel + hipBLASLt")
     ap.add_argument("--bwd-form", choices=["stored", "recompute"], default="stored",
                     help="workloads bwd, bwd_cfg3: dS stored in scratch memory and dq streamed from it, or the scores recomputed for dq")

@@ -1,5 +1,5 @@
-// C ABI of libhstu_linear.so: layer norm and norm-multiply-concatenate kernels + hipBLASLt GEMMs with fused bias /
-// SiLU epilogues and the residual as C operand.
+// C ABI of libhstu_linear.so: layer norm and norm-multiply-concatenate kernels, hipBLASLt GEMMs with fused bias /
+// SiLU epilogues and the residual as C operand, the fused q/k/v producer and the concatenating output GEMM.
 // Declarations and the reference interfaces they replace are in include/hstu_linear.h.
 #include "hstu_linear.h"
 
@@ -246,19 +246,33 @@ int output_blocks(const HstuOutputArgs* a) {
     return 1 + (a->concat_u ? 1 : 0) + (a->concat_x ? 1 : 0);
 }
 
+int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hipStream_t stream);
+
+// path = 2: which shapes the concatenating GEMM kernel takes, and what the norm-multiply kernel has to leave for it.
 bool output_fused_shape(const HstuOutputArgs* a) {
     const int64_t d = (int64_t)a->heads * a->linear_dim;
-    if (a->d_out != hstu::kOutCols || d < 32 || d > 1024 || (d & 31) != 0 || (a->dtype != 0 && a->dtype != 1)) return false;
-    if (a->group_norm) {
-        const int gl = a->linear_dim / 8;
-        if (a->linear_dim < 32 || (a->linear_dim & 7) != 0 || (gl & (gl - 1)) != 0 || a->heads > hstu::kOutMaxHeads) return false;
-    }
+    if (a->d_out != hstu::kOutCols || d < 64 || d > 4096 || (d & 63) != 0 || (a->dtype != 0 && a->dtype != 1)) return false;
+    if (a->group_norm && a->silu_u && a->concat_u && a->concat_x) return false;  // (SiLU(u) as a block of its own: layer norm only)
+    if (a->attn_row_stride >= (1 << 22) || a->u_row_stride >= (1 << 22)) return false;  // 32-bit byte offsets within a row block
     return true;
 }
 
-template <class TT, bool GROUP>
-int launch_output_fused_t(const hstu::OutputFusedParams& p, hipStream_t stream) {
-    auto kern = hstu::hstu_output_fused_kernel<TT, GROUP>;
+// The copy of u goes through SiLU: then it is written beside y, as a matrix of its own.
+bool output_fused_u_made(const HstuOutputArgs* a) { return !a->group_norm && a->concat_u && a->silu_u; }
+
+// path = 0: the concatenating path where it applies and the rows fill the chip (a workgroup takes 256 of them).
+bool output_takes_fused(const HstuOutputArgs* a) {
+    return a->path == 2 || (a->path == 0 && a->rows >= 4096 && output_fused_shape(a));
+}
+
+size_t output_fused_workspace(const HstuOutputArgs* a) {
+    const size_t d = (size_t)a->heads * a->linear_dim;
+    return ((size_t)a->rows * d * 2 * (output_fused_u_made(a) ? 2 : 1) + 255) & ~(size_t)255;
+}
+
+template <class TT>
+int launch_output_gemm_t(const hstu::OutputGemmParams& p, hipStream_t stream) {
+    auto kern = hstu::hstu_output_gemm_kernel<TT>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, hstu::kOutLds);
@@ -268,37 +282,37 @@ int launch_output_fused_t(const hstu::OutputFusedParams& p, hipStream_t stream) 
         }
         attr_done = true;
     }
-    const long long grid = (p.rows + hstu::kOutRows - 1) / hstu::kOutRows;
+    const long long grid = hstu::output_gemm_grid(p.rows);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(hstu::kOutWaves * 64), hstu::kOutLds, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
-        snprintf(g_last_error, sizeof(g_last_error), "fused output kernel launch: %s", hipGetErrorString(e));
+        snprintf(g_last_error, sizeof(g_last_error), "output GEMM kernel launch: %s", hipGetErrorString(e));
         return -7;
     }
     return 0;
 }
 
-// The caller has checked output_fused_shape(a) and the pointers of x, output_weight, out.
+// The caller has checked output_fused_shape(a), the pointers of x, output_weight, out and the size of the workspace.
+// y (and SiLU(u) where it is a block) go to the workspace; u and attn are read by the GEMM where they are.
 int launch_output_fused(const HstuOutputArgs* a, hipStream_t stream) {
     const int d = a->heads * a->linear_dim;
-    if (a->attn_row_stride < d || a->u_row_stride < d) return -5;
-    if (((a->attn_row_stride | a->u_row_stride) & 7) != 0) return -4;
-    if (a->mul_u_activation < 0 || a->mul_u_activation > 2) return -5;
-    if (!a->attn || !a->u || !a->norm_weight || !a->norm_bias) return -1;
-    if ((((uintptr_t)a->attn | (uintptr_t)a->u) & 15) != 0) return -4;
-    if (!a->group_norm && (((uintptr_t)a->norm_weight | (uintptr_t)a->norm_bias) & 15) != 0) return -4;
+    const bool u_made = output_fused_u_made(a);
     const int blocks = output_blocks(a);
-    hstu::OutputFusedParams p;
-    p.attn = (const char*)a->attn, p.u = (const char*)a->u, p.x = (const char*)a->x;
-    p.attn_rs = a->attn_row_stride, p.u_rs = a->u_row_stride, p.x_rs = a->x_row_stride;
-    p.norm_weight = (const char*)a->norm_weight, p.norm_bias = (const char*)a->norm_bias, p.eps = a->norm_eps;
-    p.w = (const char*)a->output_weight, p.out = (char*)a->out, p.rows = a->rows;
-    p.d = d, p.heads = a->heads, p.group_lanes = a->group_norm ? a->linear_dim / 8 : 0;
-    p.blk_u = (blocks == 3 || (!a->group_norm && a->concat_u)) ? 1 : 0;
-    p.blk_x = (blocks == 3 || (!a->group_norm && a->concat_x)) ? 1 : 0;
-    p.silu_u = a->silu_u ? 1 : 0, p.mul_act = a->mul_u_activation;
-    if (a->dtype == 0) return a->group_norm ? launch_output_fused_t<hstu::Bf16, true>(p, stream) : launch_output_fused_t<hstu::Bf16, false>(p, stream);
-    return a->group_norm ? launch_output_fused_t<hstu::Fp16, true>(p, stream) : launch_output_fused_t<hstu::Fp16, false>(p, stream);
+    const bool cu = blocks == 3 || (!a->group_norm && a->concat_u), cx = blocks == 3 || (!a->group_norm && a->concat_x);
+    HstuOutputArgs made = *a;
+    made.concat_u = u_made ? 1 : 0, made.concat_x = 0;
+    const int64_t ws_rs = (int64_t)d * (u_made ? 2 : 1);
+    int rc = launch_norm_mul(&made, a->workspace, ws_rs, stream);
+    if (rc != 0) return rc;
+    hstu::OutputGemmParams p;
+    int n = 0;
+    if (cu) p.src[n] = u_made ? (const char*)a->workspace : (const char*)a->u, p.src_rs[n] = u_made ? ws_rs : a->u_row_stride, ++n;
+    if (cx) p.src[n] = (const char*)a->attn, p.src_rs[n] = a->attn_row_stride, ++n;
+    p.src[n] = (const char*)a->workspace + (u_made ? (int64_t)d * 2 : 0), p.src_rs[n] = ws_rs, ++n;
+    for (int i = n; i < 3; ++i) p.src[i] = p.src[0], p.src_rs[i] = p.src_rs[0];
+    p.nsrc = n, p.d = d;
+    p.x = (const char*)a->x, p.x_rs = a->x_row_stride, p.w = (const char*)a->output_weight, p.out = (char*)a->out, p.rows = a->rows;
+    return a->dtype == 0 ? launch_output_gemm_t<hstu::Bf16>(p, stream) : launch_output_gemm_t<hstu::Fp16>(p, stream);
 }
 
 int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hipStream_t stream) {
@@ -641,7 +655,7 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
 
 size_t hstu_output_workspace_bytes(const HstuOutputArgs* a) {
     if (!a || a->rows <= 0 || a->heads <= 0 || a->linear_dim <= 0) return 0;
-    if (a->path == 2) return 0;
+    if (output_takes_fused(a)) return output_fused_shape(a) ? output_fused_workspace(a) : 0;
     return joined_bytes(a) + kGemmScratch;
 }
 
@@ -662,11 +676,15 @@ int hstu_output_forward(const HstuOutputArgs* a, void* stream_) {
     if ((((uintptr_t)a->x | (uintptr_t)a->output_weight | (uintptr_t)a->out) & 15) != 0) return -4;
     hipStream_t stream = (hipStream_t)stream_;
     if (a->path == 2 && !output_fused_shape(a)) {
-        snprintf(g_last_error, sizeof(g_last_error), "the fused output kernel takes d_out = 512, heads * linear_dim a multiple of 32 up "
-                 "to 1024 and, with group norm, linear_dim a power of two >= 32 and at most 8 heads");
+        snprintf(g_last_error, sizeof(g_last_error), "the concatenating output kernel takes d_out = 512 and heads * linear_dim a multiple "
+                 "of 64 up to 4096, row strides below 2^22 (and, with group norm, no SiLU on a copied u)");
         return -6;
     }
-    if (a->path == 2) return launch_output_fused(a, stream);
+    if (output_takes_fused(a)) {
+        if (!a->workspace) return -1;
+        if ((size_t)a->workspace_bytes < output_fused_workspace(a) || ((uintptr_t)a->workspace & 255) != 0) return -4;
+        return launch_output_fused(a, stream);
+    }
     if (!a->workspace) return -1;
     if ((size_t)a->workspace_bytes < joined_bytes(a) + kGemmScratch || ((uintptr_t)a->workspace & 255) != 0) return -4;
     const int k = output_blocks(a) * a->heads * a->linear_dim;

@@ -1,222 +1,143 @@
-// Fused consumer of the attention output for gfx950: norm(attn) * act(u), the optional copies of u and attn beside it,
-// the output projection and the residual in one kernel -- `joined` never exists in memory.
+// Output projection of the attention block for gfx950 with the concatenation folded in:
 //
-//     out[r, :] = x[r, :] + [u' | attn | y][r, :] @ W,     y = act(u) * norm(attn)
-// (hstu_compute_output of the reference, ops/hstu_compute.py:107-214, in its forward, dropout-free form
-// ops/pytorch/pt_hstu_linear.py:24-124; which blocks exist and what u' is: see HstuOutputArgs.)
+//     out[r, :] = x[r, :] + [s0 | s1 | s2][r, :] @ W
 //
-// A workgroup of 8 waves owns 128 rows and all 512 output columns: wave (rh, cb) accumulates rows rh*64 .. +64 times
-// columns cb*128 .. +128 (2 x 4 MFMA blocks of 32 x 32, 128 accumulator registers).  The depth K = blocks * d is
-// walked in tiles of 32.  Per tile
-//   * W[32 k, 512 n] (32 KB) is copied HBM/L2 -> LDS with global_load_lds_dwordx4 two tiles ahead (three slots), laid
-//     out as four slabs of 128 columns in the format of the q/k/v producer (256-byte rows, chunk swizzle swz_w) and
-//     read transposed (ds_read_b64_tr_b16) as the A operand of  C^T[n, r] += W^T[n, k] . joined^T[k, r];
-//   * the 128 x 32 slice of `joined` (8 KB) is MADE by the workgroup: every thread loads 8 elements of attn and of u
-//     one tile ahead, turns them into 8 elements of u', attn or y (statistics of the row from a pass over the
-//     workgroup's attn rows at the start, kept in LDS) and writes them to one of three LDS slots, from where the waves
-//     read their B operands (ds_read_b128, lane = row).
-// One barrier per tile.  The epilogue turns the fp32 accumulators around in LDS (the W ring is dead by then), adds the
-// residual row-contiguously in fp32, rounds once and stores whole 128-byte lines.
-// HBM traffic: attn, u, x read once (u and attn again from L2 for their copies), out written once; W (K x 512, at most
-// 3 MB) stays in every XCD's L2.
+// where the up to three column blocks of the left operand are separate matrices (u or SiLU(u), attn, and
+// y = act(u) * norm(attn) as the norm-multiply kernel leaves it): `joined` of the reference (hstu_compute_output,
+// ops/hstu_compute.py:107-214; ops/pytorch/pt_hstu_linear.py:87-124) is never written, two of its three blocks are
+// read where they already are.
+//
+// A workgroup of 4 waves, one per SIMD, owns 256 rows and 256 of the 512 output columns: wave (rh, cw) accumulates rows
+// rh*128 .. +128 times columns cw*128 .. +128 of them, 4 x 4 MFMA blocks of 32 x 32 in 256 accumulator registers, so
+// that an operand read from LDS feeds four MFMAs (half a KB of LDS reads per MFMA).  The two workgroups of a row block
+// run one after the other on the same XCD, so the second finds the rows in that XCD's L2.
+// The depth K = blocks * d is walked in tiles of 32.  Both operands come into LDS with global_load_lds_dwordx4 and
+// nothing else touches them: W[32 k, 256 n] per tile (16 KB, two slabs of 128 columns in the format of the q/k/v
+// producer, read transposed with ds_read_b64_tr_b16 as the A operand of  C^T[n, r] += W^T[n, k] . rows^T[k, r]) in
+// a ring of four, issued two tiles before use; the rows in slices of two tiles (256 x 64, 32 KB: whole 128-byte
+// lines, the eight chunks of a row swizzled with row / 2, read with ds_read_b128 as the B operand, lane = row) in a
+// ring of three, issued two and a half slices before use: with one wave per SIMD nothing but the depth of these rings
+// hides the latency of L2 and HBM, and a tile lasts only half a microsecond.  One barrier per tile, between its two
+// 16-deep steps, with the operands of the step behind it already in registers.  Every step is 16 MFMAs with exactly
+// one memory instruction behind each (12 operand reads for the next step, 4 copy instructions): issued in bursts,
+// the same instructions hold up the MFMA behind them and the kernel runs as the sum of its parts.  The epilogue turns
+// the fp32 accumulators around in LDS (the rings are dead by then), adds the residual row-contiguously in fp32,
+// rounds once and stores whole 128-byte lines.
 #pragma once
+#include <type_traits>
+
 #include "hstu_common.h"
 #include "hstu_uqvk_kernel.h"
 
 namespace hstu {
 
-struct OutputFusedParams {
-    const char* attn;
-    const char* u;
-    const char* x;
-    int64_t attn_rs, u_rs, x_rs;  // elements
-    const char* norm_weight;
-    const char* norm_bias;
-    float eps;
-    const char* w;  // [K, 512] row-major
-    char* out;      // [rows, 512] dense
+struct OutputGemmParams {
+    const char* src[3];  // the column blocks of the left operand, [rows, d] each
+    int64_t src_rs[3];   // their row strides, elements
+    int nsrc;            // 1 .. 3
+    int d;               // columns per block: a multiple of 32
+    const char* x;       // residual [rows, 512]
+    int64_t x_rs;
+    const char* w;       // [nsrc * d, 512] row-major
+    char* out;           // [rows, 512] dense
     int64_t rows;
-    int d;           // heads * linear_dim: multiple of 32, at most 1024
-    int heads;       // group norm: at most 8
-    int group_lanes; // group norm: linear_dim / 8 (a power of two, at least 4); 0 = layer norm
-    int blk_u, blk_x;  // 1: the copy of u (first) / of attn (before y) is part of `joined`
-    int silu_u;      // layer norm: the copied u goes through SiLU; group norm: u does before both uses
-    int mul_act;     // layer norm: 0 none, 1 sigmoid, 2 SiLU on the u that multiplies
 };
 
-constexpr int kOutWaves = 8, kOutRows = 128, kOutCols = 512, kOutTileK = 32;
-constexpr int kOutWSlot = kOutTileK * kOutCols * 2;  // 32 KB
-constexpr int kOutASlot = kOutRows * kOutTileK * 2;  // 8 KB
-constexpr int kOutMaxHeads = 8;
-constexpr int kOutStats = kOutRows * kOutMaxHeads * 8;
-constexpr int kOutLds = 3 * kOutWSlot + 3 * kOutASlot + kOutStats;
-constexpr int kOutStageRow = 64 * 4 + 16;  // staging row: 64 fp32 outputs + pad
+constexpr int kOutWaves = 4, kOutRows = 256, kOutCols = 512, kOutWgCols = 256, kOutTileK = 32;
+constexpr int kOutSliceK = 64;                          // the rows come in slices of two tiles: whole 128-byte lines
+constexpr int kOutWSlot = kOutTileK * kOutWgCols * 2;  // 16 KB
+constexpr int kOutASlot = kOutRows * kOutSliceK * 2;   // 32 KB
+constexpr int kOutWRing = 4, kOutARing = 3;
+constexpr int kOutLds = kOutWRing * kOutWSlot + kOutARing * kOutASlot;
+constexpr int kOutStageRow = 64 * 4 + 16;  // staging row of the epilogue: 64 fp32 outputs + pad
 
-__device__ __forceinline__ float out_sigmoid(float v) { return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * v)); }
+// Workgroups b and b + 8 land on the same XCD one after the other: they take the two column halves of one row block.
+__host__ __device__ inline long long output_gemm_grid(long long rows) {
+    const long long row_blocks = (rows + kOutRows - 1) / kOutRows;
+    return (row_blocks + 7) / 8 * 16;
+}
 
-template <class TT, bool GROUP>
-__global__ __launch_bounds__(kOutWaves * 64, 2) void hstu_output_fused_kernel(const OutputFusedParams p) {
+// Wait until at most N of the wave's copies into LDS are outstanding (they complete in order), then the barrier.
+template <int N>
+__device__ __forceinline__ void out_step_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
+}
+
+template <class TT>
+__global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(const OutputGemmParams p) {
     typedef typename TT::vec8 vec8;
     typedef typename TT::elem elem;
-    constexpr int NPW = (kOutWSlot / 1024) / kOutWaves;  // W copy instructions per wave and tile: 4
-    constexpr int PD = 3;
+    constexpr int NPW = (kOutWSlot / 1024) / kOutWaves;  // copy instructions per wave and 16 KB tile: 4
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    char* const a_ring = smem + 3 * kOutWSlot;
-    float* const stats = (float*)(smem + 3 * kOutWSlot + 3 * kOutASlot);  // [row][head] -> (mean, rstd)
+    char* const a_ring = smem + kOutWRing * kOutWSlot;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 5, l32 = lane & 31;
-    const int rh = wave >> 2, cb = wave & 3;
-    const int64_t row0 = (int64_t)blockIdx.x * kOutRows;
-    const int tpb = p.d / kOutTileK;             // tiles per block of `joined`
-    const int nblocks = p.blk_u + p.blk_x + 1;
-    const int ntiles = nblocks * tpb;
+    const int rh = wave >> 1, cw = wave & 1;
+    const unsigned pair = blockIdx.x >> 3;
+    const int colhalf = pair & 1;
+    const int64_t row0 = ((int64_t)(pair >> 1) * 8 + (blockIdx.x & 7)) * kOutRows;
+    if (row0 >= p.rows) return;
+    const int tpb = p.d / kOutTileK;  // tiles per block
+    const int ntiles = p.nsrc * tpb;
+    const int nslices = ntiles / 2;
 
-    // ---- W copies: instruction i of this wave moves chunks (wave + 8 i) * 64 + lane of the tile (slab, k row, chunk)
+    // ---- W copies: instruction i of this wave moves chunks (wave + 4 i) * 64 + lane of the tile (slab, k row, chunk)
     unsigned coff[NPW];
 #pragma unroll
     for (int i = 0; i < NPW; ++i) {
         const int pidx = (wave + kOutWaves * i) * 64 + lane;
         const int slab = pidx >> 9, row = (pidx >> 4) & 31;
         const int logical = (pidx & 15) ^ swz_w(row);
-        coff[i] = (unsigned)row * (unsigned)(kOutCols * 2) + slab * 256 + logical * 16;
+        coff[i] = (unsigned)row * (unsigned)(kOutCols * 2) + (colhalf * 2 + slab) * 256 + logical * 16;
     }
-    auto issue_w = [&](int t) {
-        char* slot = smem + (t % 3) * kOutWSlot;
-        const char* src = p.w + (int64_t)t * kOutTileK * kOutCols * 2;
-#pragma unroll
-        for (int i = 0; i < NPW; ++i) global_load_lds16_soff(src, coff[i], slot + (wave + kOutWaves * i) * 1024);
+    // (past the end: the last tile again, into a slot nobody reads -- the number of copies in flight is what the
+    // waits count)
+    int tw = 0;  // the W tile the next copy is for
+    // (one instruction of the four at a time: they are issued between MFMAs)
+    auto issue_w = [&](int i, int slot) __attribute__((always_inline)) {
+        const int tc = tw < ntiles ? tw : ntiles - 1;
+        const char* src = p.w + (int64_t)tc * kOutTileK * kOutCols * 2;
+        global_load_lds16_soff(src, coff[i], smem + slot * kOutWSlot + (wave + kOutWaves * i) * 1024);
+        if (i == NPW - 1) ++tw;
     };
-    issue_w(0);
-    if (ntiles > 1) issue_w(1);
-
-    // ---- statistics of this workgroup's attn rows: wave w takes rows 16 w .. +16, a lane chunks lane and lane + 64
-    {
-        const int chunks = p.d >> 3;
-        for (int i = 0; i < 16; ++i) {
-            const int lr = wave * 16 + i;
-            int64_t r = row0 + lr;
-            r = r < p.rows ? r : p.rows - 1;
-            float v[2][8];
-            float sum[2] = {0.f, 0.f};
+    // ---- slice copies: a slice is 256 rows x 64 columns, 128-byte rows whose eight 16-byte chunks are swizzled with
+    // the row; instruction i of this wave brings the 1 KB at byte (wave + 4 i) * 1024 of the slot, i.e. rows
+    // (wave + 4 i) * 8 + lane / 8, physical chunk lane % 8, which holds the logical chunk lc
+    const int lc = (lane & 7) ^ (((wave & 1) * 4 + (lane >> 4)) & 7);  // chunk ^ (row / 2) % 8
+    // (the offsets of the block in progress: recomputed when the block changes, not picked from a table, which the
+    // compiler would keep in scratch memory and wait for before every copy)
+    int rrel[8];
 #pragma unroll
-            for (int c2 = 0; c2 < 2; ++c2) {
-                const int c = lane + 64 * c2;
-                if (c < chunks) {
-                    const vec8 raw = *(const vec8*)(p.attn + (r * p.attn_rs + (int64_t)c * 8) * 2);
+    for (int i = 0; i < 8; ++i) {
+        int64_t r = row0 + (wave + kOutWaves * i) * 8 + (lane >> 3);
+        r = r < p.rows ? r : p.rows - 1;  // rows past the end repeat the last one; they are never stored
+        rrel[i] = (int)(r - row0);
+    }
+    int sb = 0, scol = 0, sn = 0;
+    unsigned soff[8];
+    const char* sbase;
+    auto set_block = [&]() __attribute__((always_inline)) {
+        const int64_t rs = sb == 0 ? p.src_rs[0] : (sb == 1 ? p.src_rs[1] : p.src_rs[2]);
+        const char* s0 = sb == 0 ? p.src[0] : (sb == 1 ? p.src[1] : p.src[2]);
+        sbase = s0 + row0 * rs * 2;
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        v[c2][j] = (float)raw[j];
-                        sum[c2] += v[c2][j];
-                    }
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) v[c2][j] = 0.f;
-                }
-            }
-            if constexpr (GROUP) {
-                const float inv_n = 1.0f / (float)(p.group_lanes * 8);
-#pragma unroll
-                for (int c2 = 0; c2 < 2; ++c2) {
-                    const int c = lane + 64 * c2;
-                    float s1 = sum[c2];
-                    for (int dd = 1; dd < p.group_lanes; dd <<= 1) s1 += __shfl_xor(s1, dd, 64);
-                    const float mean = s1 * inv_n;
-                    float sq = 0.f;
-                    if (c < chunks)
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) sq += (v[c2][j] - mean) * (v[c2][j] - mean);
-                    for (int dd = 1; dd < p.group_lanes; dd <<= 1) sq += __shfl_xor(sq, dd, 64);
-                    if (c < chunks && (c & (p.group_lanes - 1)) == 0) {
-                        const int head = c / p.group_lanes;
-                        stats[(lr * kOutMaxHeads + head) * 2] = mean;
-                        stats[(lr * kOutMaxHeads + head) * 2 + 1] = __builtin_amdgcn_rsqf(sq * inv_n + p.eps);
-                    }
-                }
-            } else {
-                const float inv_n = 1.0f / (float)p.d;
-                float s1 = sum[0] + sum[1];
-#pragma unroll
-                for (int dd = 32; dd >= 1; dd >>= 1) s1 += __shfl_xor(s1, dd, 64);
-                const float mean = s1 * inv_n;
-                float sq = 0.f;
-#pragma unroll
-                for (int c2 = 0; c2 < 2; ++c2)
-                    if (lane + 64 * c2 < chunks)
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) sq += (v[c2][j] - mean) * (v[c2][j] - mean);
-#pragma unroll
-                for (int dd = 32; dd >= 1; dd >>= 1) sq += __shfl_xor(sq, dd, 64);
-                if (lane == 0) {
-                    stats[lr * kOutMaxHeads * 2] = mean;
-                    stats[lr * kOutMaxHeads * 2 + 1] = __builtin_amdgcn_rsqf(sq * inv_n + p.eps);
-                }
+        for (int i = 0; i < 8; ++i) soff[i] = (unsigned)rrel[i] * (unsigned)(rs * 2) + lc * 16;
+    };
+    set_block();
+    // (one instruction of the eight at a time)
+    auto issue_slice = [&](int i, int slot) __attribute__((always_inline)) {
+        global_load_lds16_soff(sbase + scol, soff[i], a_ring + slot * kOutASlot + (wave + kOutWaves * i) * 1024);
+        if (i == 7 && ++sn < nslices) {  // (past the end: the last slice again)
+            scol += kOutSliceK * 2;
+            if (scol == p.d * 2) {
+                scol = 0, sb = sb + 1 < p.nsrc ? sb + 1 : 0;
+                set_block();
             }
         }
-    }
-
-    // ---- the slice of `joined` a thread makes per tile: row tid / 4, eight columns (tid % 4) * 8 .. of the tile
-    const int arow = tid >> 2, achunk = tid & 3;
-    int64_t arow_g = row0 + arow;
-    arow_g = arow_g < p.rows ? arow_g : p.rows - 1;  // rows past the end repeat the last one; they are never stored
-    const char* attn_row = p.attn + arow_g * p.attn_rs * 2 + achunk * 16;
-    const char* u_row = p.u + arow_g * p.u_rs * 2 + achunk * 16;
-    char* const a_dst = a_ring + arow * 64 + ((achunk ^ ((arow >> 2) & 3)) * 16);
-    vec8 raw_a, raw_u;
-    auto load_raw = [&](int t) __attribute__((always_inline)) {
-        const int col = (t % tpb) * kOutTileK;
-        raw_a = *(const vec8*)(attn_row + col * 2);
-        raw_u = *(const vec8*)(u_row + col * 2);
     };
-    auto make_a = [&](int t) __attribute__((always_inline)) {
-        const int b = t / tpb;
-        const int col = (t - b * tpb) * kOutTileK + achunk * 8;
-        vec8 o;
-        if (p.blk_u && b == 0) {  // u' : the copy of u
-            o = raw_u;
-            if (p.silu_u) {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float uf = (float)raw_u[j];
-                    o[j] = (elem)(uf * out_sigmoid(uf));
-                }
-            }
-        } else if (p.blk_x && b == p.blk_u) {  // the copy of attn
-            o = raw_a;
-        } else {  // y
-            const int head = GROUP ? col / (p.group_lanes * 8) : 0;
-            const float mean = stats[(arow * kOutMaxHeads + head) * 2], rstd = stats[(arow * kOutMaxHeads + head) * 2 + 1];
-            float wv[8], bv[8];
-            if constexpr (GROUP) {
-                const float w1 = (float)((const elem*)p.norm_weight)[head], b1 = (float)((const elem*)p.norm_bias)[head];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) wv[j] = w1, bv[j] = b1;
-            } else {
-                const vec8 w8 = *(const vec8*)(p.norm_weight + col * 2), b8 = *(const vec8*)(p.norm_bias + col * 2);
-#pragma unroll
-                for (int j = 0; j < 8; ++j) wv[j] = (float)w8[j], bv[j] = (float)b8[j];
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float uf = (float)raw_u[j];
-                float mul = uf;
-                if constexpr (GROUP) {
-                    if (p.silu_u) mul = uf * out_sigmoid(uf);
-                } else {
-                    if (p.mul_act == 1) mul = out_sigmoid(uf);
-                    if (p.mul_act == 2) mul = uf * out_sigmoid(uf);
-                }
-                o[j] = (elem)(mul * (((float)raw_a[j] - mean) * rstd * wv[j] + bv[j]));
-            }
-        }
-        *HSTU_LDS(vec8, a_dst + (t % 3) * kOutASlot) = o;
-    };
-    load_raw(0);
-    __syncthreads();  // the statistics are there
-    make_a(0);
-    if (ntiles > 1) load_raw(1);
 
     // ---- operand addresses
     int waddr[2][4];  // transposing reads of a W slab: lane supplies the address of 4 consecutive n of k row 8g + 4sec + j
@@ -228,68 +149,114 @@ __global__ __launch_bounds__(kOutWaves * 64, 2) void hstu_output_fused_kernel(co
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) {
                 const int chunk = dt * 4 + 2 * half + (q4 >> 1);
-                waddr[sec][dt] = cb * (32 * 256) + row * 256 + ((chunk ^ swz_w(row)) * 16) + (q4 & 1) * 8;
+                waddr[sec][dt] = cw * (32 * 256) + row * 256 + ((chunk ^ swz_w(row)) * 16) + (q4 & 1) * 8;
             }
         }
     }
-    int baddr[2][2];  // B operands: row rh*64 + rb*32 + l32 of the slice, columns 16 ks + 8 g .. +8
+    int baddr[2][2];  // B operands: row rh*128 + rb*32 + l32 of the slice, columns 32 half + 16 ks + 8 g .. +8
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const int row = rh * 64 + rb * 32 + l32;
-            baddr[rb][ks] = row * 64 + (((ks * 2 + g) ^ ((row >> 2) & 3)) * 16);
+            const int row = rh * 128 + l32;
+            baddr[half][ks] = row * 128 + (((half * 4 + ks * 2 + g) ^ ((row >> 1) & 7)) * 16);
         }
 
-    f32x16_t acc[2][4];
+    f32x16_t acc[4][4];
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[rb][dt][r] = 0.f;
 
-    for (int t = 0; t < ntiles; ++t) {
-        // W(t) has landed for this wave (what may still be in flight was issued after it: the copies of W(t+1) and the
-        // loads for slice t+1), this thread's part of slice t is written ...
-        if (t + 1 >= ntiles) __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-        else __builtin_amdgcn_s_waitcnt(0x0070 | (NPW + 2));
-        __syncthreads();  // ... and so for every wave; nobody reads tile t - 1 any more, whose slots tile t + 2 takes
-        // slice t + 1 first: its loads were the last thing issued a tile ago, so waiting for them waits for nothing newer
-        if (t + 1 < ntiles) make_a(t + 1);
-        if (t + 2 < ntiles) issue_w(t + 2);
-        if (t + 2 < ntiles) load_raw(t + 2);
-        const char* wt = smem + (t % 3) * kOutWSlot;
-        const char* at = a_ring + (t % 3) * kOutASlot;
-        vec8 breg[2][2];
+    // The operands of the step in flight and of the one after.  A step is 16 MFMAs with one memory instruction behind
+    // each: with one wave per SIMD an LDS read or a copy that is issued in a burst holds up the MFMA behind it, while
+    // one at a time they disappear behind the 32 cycles of the MFMA before.  Slots 0 .. 3: the B operands of the next
+    // step, 4 .. 11: the halves of its A operands, 12 .. 15: four copy instructions.
+    s16x4_t flo[2][4], fhi[2][4];
+    vec8 br[2][4];
+    auto read_op = [&](int j, int wslot, int aslot, int half, int ks, s16x4_t(&lo)[4], s16x4_t(&hi)[4], vec8(&b)[4]) __attribute__((always_inline)) {
+        const char* wt = smem + wslot * kOutWSlot + ks * 16 * 256;
+        if (j < 4) b[j] = *HSTU_LDS(const vec8, a_ring + aslot * kOutASlot + baddr[half][ks] + j * 4096);
+        else if (j & 1) hi[(j - 4) >> 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, wt + waddr[1][(j - 4) >> 1]));
+        else lo[(j - 4) >> 1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(HSTU_LDS(s16x4_t, wt + waddr[0][(j - 4) >> 1]));
+    };
+    auto mma = [&](int m, const s16x4_t(&lo)[4], const s16x4_t(&hi)[4], const vec8(&b)[4]) __attribute__((always_inline)) {
+        const s16x8_t both = __builtin_shufflevector(lo[m >> 2], hi[m >> 2], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc[m & 3][m >> 2] = TT::mfma(__builtin_bit_cast(vec8, both), b[m & 3], acc[m & 3][m >> 2]);
+    };
+
+    // ---- prologue: W(0 .. 2), slices 0 and 1 and the first half of slice 2, waited for once
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
+    for (int t = 0; t < 3; ++t)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) breg[rb][ks] = *HSTU_LDS(const vec8, at + baddr[rb][ks]);
-        // 8 A operands (ks, dt) = (m / 4, m % 4), each used for the wave's two row blocks, requested PD ahead
-        auto load_op = [&](int m) __attribute__((always_inline)) -> vec8 {
-            const char* b = wt + (m >> 2) * 16 * 256;
-            return read_vt_operand<TT>(b + waddr[0][m & 3], b + waddr[1][m & 3]);
-        };
-        vec8 fr[PD];
+        for (int i = 0; i < NPW; ++i) issue_w(i, t);
 #pragma unroll
-        for (int m = 0; m < PD; ++m) fr[m] = load_op(m);
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int m = 0; m < 8; ++m) {
+        for (int i = 0; i < 8; ++i) issue_slice(i, t);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) issue_slice(i, 2);
+    out_step_barrier<0>();
+#pragma unroll
+    for (int j = 0; j < 12; ++j) read_op(j, 0, 0, 0, 0, flo[0], fhi[0], br[0]);
+
+    // Tile t (half of slice t / 2).  Step A multiplies its first 16 columns, reads the operands of step B and issues the
+    // copies of W(t + 3) into the slot of tile t - 1; the barrier publishes W(t + 1) and, for even t + 1, the next
+    // slice (behind the copies of W(t + 1), issued in tile t - 2, came four copies in each of the four steps since:
+    // the wait leaves those outstanding); step B multiplies the other 16 columns, reads the operands of tile t + 1
+    // and issues half the copies of a slice: in the second tile of slice S the first half of slice S + 3 into the slot
+    // of S, which every wave has finished reading, in the tile after it the second half.
+    int wslot = 0, aslot = 0;  // t % 4, (t / 2) % 3
+    auto tile = [&](auto Oddc) __attribute__((always_inline)) {
+        constexpr bool ODD = decltype(Oddc)::value;
+        const int wslot1 = (wslot + 1) & (kOutWRing - 1), wslot3 = (wslot + 3) & (kOutWRing - 1);
+        const int aslot1 = ODD ? (aslot == kOutARing - 1 ? 0 : aslot + 1) : aslot;
+        const int aslot_prev = aslot == 0 ? kOutARing - 1 : aslot - 1;
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            mma(m, flo[0], fhi[0], br[0]);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb) acc[rb][m & 3] = TT::mfma(fr[m % PD], breg[rb][m >> 2], acc[rb][m & 3]);
-            if (m + PD < 8) fr[m % PD] = load_op(m + PD);
+            if (m < 12) read_op(m, wslot, aslot, ODD, 1, flo[1], fhi[1], br[1]);
+            else issue_w(m - 12, wslot3);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
+        out_step_barrier<16>();
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            mma(m, flo[1], fhi[1], br[1]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (m < 12) read_op(m, wslot1, aslot1, !ODD, 0, flo[0], fhi[0], br[0]);
+            else if (ODD) issue_slice(m - 12, aslot);
+            else issue_slice(m - 12 + 4, aslot_prev);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        wslot = wslot1, aslot = aslot1;
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        tile(std::false_type{});
+        tile(std::true_type{});
     }
 
-    // ---- epilogue: fp32 accumulators through this wave's staging area (the W ring is dead), + x, rounding, stores
-    __syncthreads();
+    // ---- epilogue: fp32 accumulators through this wave's staging area (the rings are dead), + x, rounding, stores
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     char* stage = smem + wave * 32 * kOutStageRow;
     const int chunk = lane & 7, rsub = lane >> 3;  // 8 lanes cover one row's 64 columns, 8 rows per instruction
+    const int col0 = colhalf * kOutWgCols + cw * 128 + chunk * 8;
+    vec8 xr[4][2][4];  // the residual of everything this lane stores, requested at once (rows past the end: the last row)
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int64_t r = row0 + rh * 128 + rb * 32 + i * 8 + rsub;
+                r = r < p.rows ? r : p.rows - 1;
+                xr[rb][hf][i] = *(const vec8*)(p.x + (r * p.x_rs + col0 + hf * 64) * 2);
+            }
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
@@ -304,19 +271,17 @@ __global__ __launch_bounds__(kOutWaves * 64, 2) void hstu_output_fused_kernel(co
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = i * 8 + rsub;
-                const int64_t r = row0 + rh * 64 + rb * 32 + row;
+                const int64_t r = row0 + rh * 128 + rb * 32 + row;
                 const f32x4_t lo = *HSTU_LDS(const f32x4_t, stage + row * kOutStageRow + chunk * 32);
                 const f32x4_t hi = *HSTU_LDS(const f32x4_t, stage + row * kOutStageRow + chunk * 32 + 16);
                 if (r < p.rows) {
-                    const int col = cb * 128 + hf * 64 + chunk * 8;
-                    const vec8 xr = *(const vec8*)(p.x + (r * p.x_rs + col) * 2);
-                    vec8 o;
+                    vec8 ov;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        o[j] = (elem)(lo[j] + (float)xr[j]);
-                        o[4 + j] = (elem)(hi[j] + (float)xr[4 + j]);
+                        ov[j] = (elem)(lo[j] + (float)xr[rb][hf][i][j]);
+                        ov[4 + j] = (elem)(hi[j] + (float)xr[rb][hf][i][4 + j]);
                     }
-                    *(vec8*)(p.out + (r * kOutCols + col) * 2) = o;
+                    *(vec8*)(p.out + (r * kOutCols + col0 + hf * 64) * 2) = ov;
                 }
             }
         }

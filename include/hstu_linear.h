@@ -73,12 +73,12 @@ int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight
  *                           joined = u | attn | y only when concat_u AND concat_x, else y alone (as the reference)
  *              silu_u     : layer norm: the copied u block goes through SiLU; group norm: u does before both uses
  *     out = x + joined @ output_weight             [rows, d_out]
- * Two paths (see `path`).  Library path (the default, any shape): the norm / multiply / concatenate step is one
- * hand-written kernel (one wave per row, HBM-bound) that writes `joined` in the inputs' type; the product with the
- * residual as the GEMM's C operand runs on hipBLASLt.  Fused path (on request): one hand-written kernel in which a
- * workgroup makes its 128 x 32 slices of `joined` in LDS, tile by tile, and multiplies them with the weight tiles
- * streaming through LDS; attn, u, x are read and out is written once and nothing else touches HBM -- but at the
- * benchmark's shape it takes 1.56 ms against the library path's 1.39, which is why it is not the default.
+ * Two paths (see `path`).  Library path (any shape): the norm / multiply / concatenate step is one hand-written kernel
+ * (one wave per row, HBM-bound) that writes `joined` in the inputs' type; the product with the residual as the GEMM's
+ * C operand runs on hipBLASLt.  Concatenating path (d_out = 512): the same norm-multiply kernel writes y alone (and
+ * SiLU(u) where that is a block of `joined`), and a hand-written GEMM kernel reads the blocks of `joined` where they
+ * are -- u and attn in the caller's tensors, y in the workspace -- so that `joined` is never written: 1.17 ms against
+ * the library path's 1.39 ms at the benchmark's shape (524288 rows, 3 x 512 -> 512).
  */
 enum { HSTU_MUL_U_NONE = 0, HSTU_MUL_U_SIGMOID = 1, HSTU_MUL_U_SILU = 2 };
 
@@ -100,13 +100,13 @@ typedef struct HstuOutputArgs {
     int32_t concat_u, concat_x, group_norm, silu_u;  /* 0 / 1 */
     int32_t mul_u_activation;  /* HSTU_MUL_U_*; layer norm only */
     int32_t dtype;             /* 0 = bf16, 1 = fp16 */
-    void* workspace;           /* hstu_output_workspace_bytes() bytes, 256-byte aligned: `joined` and the GEMM's scratch
-                                  (library path only; may be NULL when that function returns 0) */
+    void* workspace;           /* hstu_output_workspace_bytes() bytes, 256-byte aligned: library path: `joined` and the
+                                  GEMM's scratch; concatenating path: y (and SiLU(u)) */
     int64_t workspace_bytes;
-    int32_t path;              /* 0 or 1 = library path (norm-mul kernel + hipBLASLt); 2 = fused kernel (norm, multiply,
-                                  concatenation, product and residual in one pass, `joined` never written): needs d_out
-                                  = 512, heads * linear_dim a multiple of 32 up to 1024 and, for group norm, linear_dim a
-                                  power of two >= 32 with at most 8 heads, else status -6 */
+    int32_t path;              /* 1 = library path (norm-mul kernel + hipBLASLt); 2 = concatenating path (norm-mul kernel
+                                  + hand-written GEMM over the blocks where they are): needs d_out = 512 and heads *
+                                  linear_dim a multiple of 64 (and, with group norm, no SiLU on a copied u), else status
+                                  -6; 0 = the concatenating path where it applies and rows >= 4096, else the library */
 } HstuOutputArgs;
 
 size_t hstu_output_workspace_bytes(const HstuOutputArgs* args);

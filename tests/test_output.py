@@ -178,7 +178,7 @@ def test_compute_output(pkg, dev, N, H, ld, D, cu, cx, act, group_norm, dtype):
 
 
 FUSED_CASES = [
-    # N, H, linear_dim, concat_u, concat_x, act, group_norm; d_model is 512, the width the fused kernel is built for
+    # N, H, linear_dim, concat_u, concat_x, act, group_norm; d_model is 512, the width the concatenating GEMM kernel is built for
     (4099, 4, 128, True, True, "none", False),
     (1000, 4, 128, False, True, "silu", False),
     (1000, 4, 128, True, False, "sigmoid", False),
@@ -194,8 +194,8 @@ FUSED_CASES = [
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("N,H,ld,cu,cx,act,group_norm", FUSED_CASES)
 def test_compute_output_fused_kernel(pkg, dev, N, H, ld, cu, cx, act, group_norm, dtype):
-    """``path=2``: norm, multiply, concatenation, product and residual in one kernel; same bar as the library path, and
-    the two paths agree with each other."""
+    """``path=2``: the norm-multiply kernel writes y alone, a hand-written GEMM reads u and attn where they are; same bar
+    as the library path, and the two paths agree with each other."""
     D = 512
     print(f"[case] fused output {N} {H} {ld} {cu} {cx} {act} group={group_norm} {dtype}", flush=True)
     blocks = _blocks(cu, cx, group_norm)
@@ -208,6 +208,54 @@ def test_compute_output_fused_kernel(pkg, dev, N, H, ld, cu, cx, act, group_norm
     kw = dict(concat_u=cu, concat_x=cx, mul_u_activation_type=act, group_norm=group_norm, num_heads=H, linear_dim=ld)
     _close(got, O.compute_output(attn, u, x, nw, nb, w, 1e-6, **kw), "fused out vs fp32 oracle")
     _close(got, lib.float().cpu(), "fused out vs library path")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N", [5000, 257])
+def test_compute_output_concat_gemm_on_views_of_wider_buffers(pkg, dev, N):
+    """u as the column slice of a [N, 4 * 512] buffer (what the producer leaves), attn as a slice of a padded one: the
+    GEMM kernel reads them through their row strides.  N = 5000 also takes this path when none is asked for."""
+    print(f"[case] concat-gemm output on strided views N={N}", flush=True)
+    H, ld, D = 4, 128, 512
+    attn, u, x, nw, nb, w = _inputs(77 + N, N, H, ld, D, 3, False, torch.bfloat16)
+    uvqk = torch.zeros(N, 4 * H * ld, dtype=torch.bfloat16, device=dev)
+    uvqk[:, : H * ld] = u.to(dev)
+    padded = torch.zeros(N, H * ld + 64, dtype=torch.bfloat16, device=dev)
+    padded[:, 32 : 32 + H * ld] = attn.to(dev)
+    u_view, attn_view = uvqk[:, : H * ld], padded[:, 32 : 32 + H * ld]
+    args = (attn_view, u_view, x.to(dev), nw.to(dev), nb.to(dev), 1e-6, w.to(dev), H, ld, 0.0, False, True, True, "none", False, False)
+    got = pkg.hstu_compute_output(*args, path=2)
+    auto = pkg.hstu_compute_output(*args)
+    lib = pkg.hstu_compute_output(*args, path=1)
+    torch.cuda.synchronize()
+    _close(got, O.compute_output(attn, u, x, nw, nb, w, 1e-6, concat_u=True, concat_x=True), "views: out vs fp32 oracle")
+    _close(got, lib.float().cpu(), "views: out vs library path")
+    assert torch.equal(auto, got if N >= 4096 else lib)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", [1, 2])
+def test_output_forward_with_silu_on_the_copied_u(dev, path):
+    """The C entry point with ``silu_u`` (the Python operator never sets it for the projection): layer norm, all three
+    blocks, SiLU(u) as the first of them -- on the concatenating path it is written beside y as a matrix of its own."""
+    import ctypes
+
+    from generative_recommenders_amd.ops import hstu_compute as hc
+
+    print(f"[case] hstu_output_forward silu_u path={path}", flush=True)
+    N, H, ld, D = 700, 4, 64, 512
+    attn, u, x, nw, nb, w = _inputs(4321, N, H, ld, D, 3, False, torch.bfloat16)
+    dv = [t.to(dev) for t in (attn, u, x, nw, nb, w)]
+    a, keep, blocks = hc._output_args(dv[0], dv[1], dv[3], dv[4], 1e-6, H, ld, True, True, "none", False, True)
+    out = torch.empty((N, D), dtype=torch.bfloat16, device=dev)
+    a.x, a.x_row_stride, a.output_weight, a.out, a.d_out, a.path = dv[2].data_ptr(), D, dv[5].data_ptr(), out.data_ptr(), D, path
+    need = hc.lib().hstu_output_workspace_bytes(ctypes.byref(a))
+    ws = torch.empty(need + 256, dtype=torch.uint8, device=dev)
+    a.workspace, a.workspace_bytes = (ws.data_ptr() + 255) & ~255, need
+    rc = hc.lib().hstu_output_forward(ctypes.byref(a), ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    torch.cuda.synchronize()
+    assert rc == 0, hc.lib().hstu_linear_last_error()
+    _close(out, O.compute_output(attn, u, x, nw, nb, w, 1e-6, silu_u=True, concat_u=True, concat_x=True), "silu_u: out vs fp32 oracle")
 
 
 @pytest.mark.gpu
