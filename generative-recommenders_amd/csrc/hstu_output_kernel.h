@@ -187,18 +187,21 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
         acc[m & 3][m >> 2] = TT::mfma(__builtin_bit_cast(vec8, both), b[m & 3], acc[m & 3][m >> 2]);
     };
 
-    // ---- prologue: W(0 .. 2), slices 0 and 1 and the first half of slice 2, waited for once
+    // ---- prologue: W(0) and slice 0 first, then W(1), W(2), slice 1 and the first half of slice 2; only the first two
+    // are waited for (every later wait leaves 16 copies outstanding, and at least 16 are issued behind each of these)
 #pragma unroll
-    for (int t = 0; t < 3; ++t)
+    for (int i = 0; i < NPW; ++i) issue_w(i, 0);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) issue_slice(i, 0);
+#pragma unroll
+    for (int t = 1; t < 3; ++t)
 #pragma unroll
         for (int i = 0; i < NPW; ++i) issue_w(i, t);
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 8; ++i) issue_slice(i, t);
+    for (int i = 0; i < 8; ++i) issue_slice(i, 1);
 #pragma unroll
     for (int i = 0; i < 4; ++i) issue_slice(i, 2);
-    out_step_barrier<0>();
+    out_step_barrier<2 * NPW + 8 + 4>();
 #pragma unroll
     for (int j = 0; j < 12; ++j) read_op(j, 0, 0, 0, 0, flo[0], fhi[0], br[0]);
 
@@ -240,8 +243,6 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
     }
 
     // ---- epilogue: fp32 accumulators through this wave's staging area (the rings are dead), + x, rounding, stores
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    char* stage = smem + wave * 32 * kOutStageRow;
     const int chunk = lane & 7, rsub = lane >> 3;  // 8 lanes cover one row's 64 columns, 8 rows per instruction
     const int col0 = colhalf * kOutWgCols + cw * 128 + chunk * 8;
     vec8 xr[4][2][4];  // the residual of everything this lane stores, requested at once (rows past the end: the last row)
@@ -255,6 +256,10 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
                 r = r < p.rows ? r : p.rows - 1;
                 xr[rb][hf][i] = *(const vec8*)(p.x + (r * p.x_rs + col0 + hf * 64) * 2);
             }
+    // the copies that are still on their way into the rings (repeats of the last tiles) have to land before the staging
+    // areas take their place; the 32 loads of the residual behind them need not
+    asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    char* stage = smem + wave * 32 * kOutStageRow;
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
