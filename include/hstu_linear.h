@@ -106,7 +106,7 @@ typedef struct HstuOutputArgs {
     int32_t path;              /* 1 = library path (norm-mul kernel + hipBLASLt); 2 = concatenating path (norm-mul kernel
                                   + hand-written GEMM over the blocks where they are): needs d_out = 512 and heads *
                                   linear_dim a multiple of 64 (and, with group norm, no SiLU on a copied u), else status
-                                  -6; 0 = the concatenating path where it applies and rows >= 4096, else the library */
+                                  -6; 0 = the concatenating path where it applies and rows >= 32768, else the library */
 } HstuOutputArgs;
 
 size_t hstu_output_workspace_bytes(const HstuOutputArgs* args);
