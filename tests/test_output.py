@@ -187,6 +187,8 @@ FUSED_CASES = [
     (333, 8, 64, True, True, "none", True),
     (129, 2, 32, True, True, "silu", False),
     (1, 8, 128, True, True, "none", False),
+    (300, 2, 32, False, False, "none", False),  # one block of 64 columns: two tiles, fewer than the rings hold
+    (70000, 2, 64, True, True, "none", False),  # more row blocks than one pass over the XCDs
 ]
 
 
