@@ -236,6 +236,34 @@ def test_compute_output_concat_gemm_on_views_of_wider_buffers(pkg, dev, N):
 
 
 @pytest.mark.gpu
+def test_compute_output_at_the_benchmark_size(pkg, dev):
+    """524288 rows, 3 x 512 -> 512 (the size of `bench.py --workload output`): the automatic choice is the concatenating
+    GEMM and it agrees with the library path everywhere; a zero weight returns the residual bit for bit (every row block
+    and both column halves are stored, none twice with different values); rows picked across the whole range, the last
+    one included, against the fp32 oracle."""
+    print("[case] output at 524288 rows", flush=True)
+    N, H, ld, D = 524288, 4, 128, 512
+    g = torch.Generator(device=dev).manual_seed(99)
+
+    def uni(*shape):
+        return (torch.rand(shape, generator=g, device=dev) * 0.2 - 0.1).to(torch.bfloat16)
+
+    attn, u, x, nw, nb, w = uni(N, H * ld), uni(N, H * ld), uni(N, D), uni(H * ld), uni(H * ld), uni(3 * H * ld, D)
+    args = (attn, u, x, nw, nb, 1e-6, w, H, ld, 0.0, False, True, True, "none", False, False)
+    auto = pkg.hstu_compute_output(*args)
+    got = pkg.hstu_compute_output(*args, path=2)
+    lib = pkg.hstu_compute_output(*args, path=1)
+    zero = pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, torch.zeros_like(w), H, ld, 0.0, False, True, True, "none", False, False, path=2)
+    torch.cuda.synchronize()
+    assert torch.equal(auto, got) and torch.equal(zero, x)
+    diff = (got.float() - lib.float())
+    assert float(diff.norm() / lib.float().norm()) <= 1e-2 and float(diff.abs().max()) <= 2e-2 * float(lib.float().abs().max())
+    rows = torch.tensor([0, 1, 255, 256, 257, 70001, 262143, 262144, 400000, N - 257, N - 2, N - 1], device=dev)
+    ref = O.compute_output(attn[rows].cpu(), u[rows].cpu(), x[rows].cpu(), nw.cpu(), nb.cpu(), w.cpu(), 1e-6, concat_u=True, concat_x=True)
+    _close(got[rows], ref, "benchmark size: sampled rows vs fp32 oracle")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("path", [1, 2])
 def test_output_forward_with_silu_on_the_copied_u(dev, path):
     """The C entry point with ``silu_u`` (the Python operator never sets it for the projection): layer norm, all three
