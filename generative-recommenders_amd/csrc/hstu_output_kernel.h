@@ -16,7 +16,7 @@
 // producer, read transposed with ds_read_b64_tr_b16 as the A operand of  C^T[n, r] += W^T[n, k] . rows^T[k, r]) in
 // a ring of four, issued two tiles before use; the rows in slices of two tiles (256 x 64, 32 KB: whole 128-byte
 // lines, the eight chunks of a row swizzled with row / 2, read with ds_read_b128 as the B operand, lane = row) in a
-// ring of three, issued two and a half slices before use: with one wave per SIMD nothing but the depth of these rings
+// ring of three, issued two slices before use: with one wave per SIMD nothing but the depth of these rings
 // hides the latency of L2 and HBM, and a tile lasts only half a microsecond.  One barrier per tile, between its two
 // 16-deep steps, with the operands of the step behind it already in registers.  Every step is 16 MFMAs with exactly
 // one memory instruction behind each (12 operand reads for the next step, 4 copy instructions): issued in bursts,
