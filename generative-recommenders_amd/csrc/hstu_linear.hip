@@ -219,19 +219,25 @@ __global__ __launch_bounds__(256) void hstu_norm_mul_kernel(NormMulParams p) {
             const int c = lane + 64 * i;
             if (c < chunks) {
                 V8 y, ucopy = uraw[i];
+                if (p.silu_u || (!GROUP && p.mul_act != HSTU_MUL_U_NONE)) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float uf = (float)uraw[i][j];
-                    const float us = uf * sigmoid_f(uf);
-                    float mul = uf;
-                    if constexpr (GROUP) {
-                        if (p.silu_u) mul = us;
-                    } else {
-                        if (p.mul_act == HSTU_MUL_U_SIGMOID) mul = sigmoid_f(uf);
-                        if (p.mul_act == HSTU_MUL_U_SILU) mul = us;
+                    for (int j = 0; j < 8; ++j) {
+                        const float uf = (float)uraw[i][j];
+                        const float us = uf * sigmoid_f(uf);
+                        float mul = uf;
+                        if constexpr (GROUP) {
+                            if (p.silu_u) mul = us;
+                        } else {
+                            if (p.mul_act == HSTU_MUL_U_SIGMOID) mul = sigmoid_f(uf);
+                            if (p.mul_act == HSTU_MUL_U_SILU) mul = us;
+                        }
+                        if (p.silu_u) ucopy[j] = (E)us;
+                        y[j] = (E)(mul * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]));
                     }
-                    if (p.silu_u) ucopy[j] = (E)us;
-                    y[j] = (E)(mul * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]));
+                } else {  // no activation anywhere: the exponentials are not worth computing to be thrown away
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        y[j] = (E)((float)uraw[i][j] * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]));
                 }
                 if (p.off_u >= 0) *(V8*)(orow + ((int64_t)p.off_u + c * 8) * 2) = ucopy;
                 if (p.off_x >= 0) *(V8*)(orow + ((int64_t)p.off_x + c * 8) * 2) = xraw[i];
