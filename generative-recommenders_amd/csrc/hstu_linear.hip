@@ -257,7 +257,8 @@ int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hi
 // path = 2: which shapes the concatenating GEMM kernel takes, and what the norm-multiply kernel has to leave for it.
 bool output_fused_shape(const HstuOutputArgs* a) {
     const int64_t d = (int64_t)a->heads * a->linear_dim;
-    if (a->d_out != hstu::kOutCols || d < 64 || d > 4096 || (d & 63) != 0 || (a->dtype != 0 && a->dtype != 1)) return false;
+    if (a->d_out < hstu::kOutWgCols || a->d_out % hstu::kOutWgCols != 0 || a->d_out > 8192) return false;
+    if (d < 64 || d > 4096 || (d & 63) != 0 || (a->dtype != 0 && a->dtype != 1)) return false;
     if (a->group_norm && a->silu_u && a->concat_u && a->concat_x) return false;  // (SiLU(u) as a block of its own: layer norm only)
     if (a->attn_row_stride >= (1 << 22) || a->u_row_stride >= (1 << 22)) return false;  // 32-bit byte offsets within a row block
     return true;
@@ -289,7 +290,7 @@ int launch_output_gemm_t(const hstu::OutputGemmParams& p, hipStream_t stream) {
         }
         attr_done = true;
     }
-    const long long grid = hstu::output_gemm_grid(p.rows);
+    const long long grid = hstu::output_gemm_grid(p.rows, p.n);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(hstu::kOutWaves * 64), hstu::kOutLds, stream, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
@@ -318,7 +319,7 @@ int launch_output_fused(const HstuOutputArgs* a, hipStream_t stream) {
     p.src[n] = (const char*)a->workspace + (u_made ? (int64_t)d * 2 : 0), p.src_rs[n] = ws_rs, ++n;
     for (int i = n; i < 3; ++i) p.src[i] = p.src[0], p.src_rs[i] = p.src_rs[0];
     p.nsrc = n, p.d = d;
-    p.x = (const char*)a->x, p.x_rs = a->x_row_stride, p.w = (const char*)a->output_weight, p.out = (char*)a->out, p.rows = a->rows;
+    p.x = (const char*)a->x, p.x_rs = a->x_row_stride, p.w = (const char*)a->output_weight, p.out = (char*)a->out, p.rows = a->rows, p.n = a->d_out;
     return a->dtype == 0 ? launch_output_gemm_t<hstu::Bf16>(p, stream) : launch_output_gemm_t<hstu::Fp16>(p, stream);
 }
 
@@ -683,7 +684,7 @@ int hstu_output_forward(const HstuOutputArgs* a, void* stream_) {
     if ((((uintptr_t)a->x | (uintptr_t)a->output_weight | (uintptr_t)a->out) & 15) != 0) return -4;
     hipStream_t stream = (hipStream_t)stream_;
     if (a->path == 2 && !output_fused_shape(a)) {
-        snprintf(g_last_error, sizeof(g_last_error), "the concatenating output kernel takes d_out = 512 and heads * linear_dim a multiple "
+        snprintf(g_last_error, sizeof(g_last_error), "the concatenating output kernel takes d_out a multiple of 256 and heads * linear_dim a multiple "
                  "of 64 up to 4096, row strides below 2^22 (and, with group norm, no SiLU on a copied u)");
         return -6;
     }

@@ -7,10 +7,10 @@
 // ops/hstu_compute.py:107-214; ops/pytorch/pt_hstu_linear.py:87-124) is never written, two of its three blocks are
 // read where they already are.
 //
-// A workgroup of 4 waves, one per SIMD, owns 256 rows and 256 of the 512 output columns: wave (rh, cw) accumulates rows
+// A workgroup of 4 waves, one per SIMD, owns 256 rows and 256 of the output columns (a multiple of 256): wave (rh, cw) accumulates rows
 // rh*128 .. +128 times columns cw*128 .. +128 of them, 4 x 4 MFMA blocks of 32 x 32 in 256 accumulator registers, so
-// that an operand read from LDS feeds four MFMAs (half a KB of LDS reads per MFMA).  The two workgroups of a row block
-// run one after the other on the same XCD, so the second finds the rows in that XCD's L2.
+// that an operand read from LDS feeds four MFMAs (half a KB of LDS reads per MFMA).  The workgroups of a row block
+// run one after the other on the same XCD, so all but the first find the rows in that XCD's L2.
 // The depth K = blocks * d is walked in tiles of 32.  Both operands come into LDS with global_load_lds_dwordx4 and
 // nothing else touches them: W[32 k, 256 n] per tile (16 KB, two slabs of 128 columns in the format of the q/k/v
 // producer, read transposed with ds_read_b64_tr_b16 as the A operand of  C^T[n, r] += W^T[n, k] . rows^T[k, r]) in
@@ -36,14 +36,15 @@ struct OutputGemmParams {
     int64_t src_rs[3];   // their row strides, elements
     int nsrc;            // 1 .. 3
     int d;               // columns per block: a multiple of 32
-    const char* x;       // residual [rows, 512]
+    const char* x;       // residual [rows, n]
     int64_t x_rs;
-    const char* w;       // [nsrc * d, 512] row-major
-    char* out;           // [rows, 512] dense
+    const char* w;       // [nsrc * d, n] row-major
+    char* out;           // [rows, n] dense
     int64_t rows;
+    int n;               // output columns: a multiple of 256
 };
 
-constexpr int kOutWaves = 4, kOutRows = 256, kOutCols = 512, kOutWgCols = 256, kOutTileK = 32;
+constexpr int kOutWaves = 4, kOutRows = 256, kOutWgCols = 256, kOutTileK = 32;
 constexpr int kOutSliceK = 64;                          // the rows come in slices of two tiles: whole 128-byte lines
 constexpr int kOutWSlot = kOutTileK * kOutWgCols * 2;  // 16 KB
 constexpr int kOutASlot = kOutRows * kOutSliceK * 2;   // 32 KB
@@ -51,10 +52,11 @@ constexpr int kOutWRing = 4, kOutARing = 3;
 constexpr int kOutLds = kOutWRing * kOutWSlot + kOutARing * kOutASlot;
 constexpr int kOutStageRow = 64 * 4 + 16;  // staging row of the epilogue: 64 fp32 outputs + pad
 
-// Workgroups b and b + 8 land on the same XCD one after the other: they take the two column halves of one row block.
-__host__ __device__ inline long long output_gemm_grid(long long rows) {
+// Workgroups b, b + 8, b + 16 ... land on the same XCD one after the other: they take the column blocks of one row
+// block (row blocks in groups of eight, one per XCD).
+__host__ __device__ inline long long output_gemm_grid(long long rows, int n) {
     const long long row_blocks = (rows + kOutRows - 1) / kOutRows;
-    return (row_blocks + 7) / 8 * 16;
+    return (row_blocks + 7) / 8 * 8 * (n / kOutWgCols);
 }
 
 // Wait until at most N of the wave's copies into LDS are outstanding (they complete in order), then the barrier.
@@ -76,9 +78,10 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 5, l32 = lane & 31;
     const int rh = wave >> 1, cw = wave & 1;
-    const unsigned pair = blockIdx.x >> 3;
-    const int colhalf = pair & 1;
-    const int64_t row0 = ((int64_t)(pair >> 1) * 8 + (blockIdx.x & 7)) * kOutRows;
+    const unsigned ncb = (unsigned)p.n / kOutWgCols;  // column blocks of a row block
+    const unsigned group = blockIdx.x / (8 * ncb), within = blockIdx.x - group * (8 * ncb);
+    const int colblk = within >> 3;
+    const int64_t row0 = ((int64_t)group * 8 + (within & 7)) * kOutRows;
     if (row0 >= p.rows) return;
     const int tpb = p.d / kOutTileK;  // tiles per block
     const int ntiles = p.nsrc * tpb;
@@ -91,7 +94,7 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
         const int pidx = (wave + kOutWaves * i) * 64 + lane;
         const int slab = pidx >> 9, row = (pidx >> 4) & 31;
         const int logical = (pidx & 15) ^ swz_w(row);
-        coff[i] = (unsigned)row * (unsigned)(kOutCols * 2) + (colhalf * 2 + slab) * 256 + logical * 16;
+        coff[i] = (unsigned)row * (unsigned)(p.n * 2) + (colblk * 2 + slab) * 256 + logical * 16;
     }
     // (past the end: the last tile again, into a slot nobody reads -- the number of copies in flight is what the
     // waits count)
@@ -99,7 +102,7 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
     // (one instruction of the four at a time: they are issued between MFMAs)
     auto issue_w = [&](int i, int slot) __attribute__((always_inline)) {
         const int tc = tw < ntiles ? tw : ntiles - 1;
-        const char* src = p.w + (int64_t)tc * kOutTileK * kOutCols * 2;
+        const char* src = p.w + (int64_t)tc * kOutTileK * p.n * 2;
         global_load_lds16_soff(src, coff[i], smem + slot * kOutWSlot + (wave + kOutWaves * i) * 1024);
         if (i == NPW - 1) ++tw;
     };
@@ -244,7 +247,7 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
 
     // ---- epilogue: fp32 accumulators through this wave's staging area (the rings are dead), + x, rounding, stores
     const int chunk = lane & 7, rsub = lane >> 3;  // 8 lanes cover one row's 64 columns, 8 rows per instruction
-    const int col0 = colhalf * kOutWgCols + cw * 128 + chunk * 8;
+    const int col0 = colblk * kOutWgCols + cw * 128 + chunk * 8;
     vec8 xr[4][2][4];  // the residual of everything this lane stores, requested at once (rows past the end: the last row)
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
@@ -286,7 +289,7 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
                         ov[j] = (elem)(lo[j] + (float)xr[rb][hf][i][j]);
                         ov[4 + j] = (elem)(hi[j] + (float)xr[rb][hf][i][4 + j]);
                     }
-                    *(vec8*)(p.out + (r * kOutCols + col0 + hf * 64) * 2) = ov;
+                    *(vec8*)(p.out + (r * p.n + col0 + hf * 64) * 2) = ov;
                 }
             }
         }

@@ -419,7 +419,7 @@ def hstu_compute_output(
     """Returns ``x + joined @ output_weight`` of shape ``[L, d_model]``.  The backward always recomputes ``joined``
     (what ``recompute_y_in_backward=True`` asks for), so the flag changes nothing.  ``path``: 1 = the norm-mul kernel
     writes ``joined`` and hipBLASLt multiplies it; 2 = the norm-mul kernel writes ``y`` alone and a hand-written GEMM
-    reads ``u`` and ``attn`` where they are (``NotImplementedError`` if the shape does not fit: d_model 512,
+    reads ``u`` and ``attn`` where they are (``NotImplementedError`` if the shape does not fit: d_model a multiple of 256,
     heads * linear_dim a multiple of 64); 0 = whichever is faster for the shape (2 where it fits and rows >= 32768)."""
     _no_dropout(dropout_ratio, training)
     torch._assert(x.dim() == 2 and x.shape[0] == attn.shape[0], "x must be 2-D with attn's row count")

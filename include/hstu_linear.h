@@ -75,7 +75,7 @@ int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight
  *     out = x + joined @ output_weight             [rows, d_out]
  * Two paths (see `path`).  Library path (any shape): the norm / multiply / concatenate step is one hand-written kernel
  * (one wave per row, HBM-bound) that writes `joined` in the inputs' type; the product with the residual as the GEMM's
- * C operand runs on hipBLASLt.  Concatenating path (d_out = 512): the same norm-multiply kernel writes y alone (and
+ * C operand runs on hipBLASLt.  Concatenating path (d_out a multiple of 256): the same norm-multiply kernel writes y alone (and
  * SiLU(u) where that is a block of `joined`), and a hand-written GEMM kernel reads the blocks of `joined` where they
  * are -- u and attn in the caller's tensors, y in the workspace -- so that `joined` is never written: 1.17 ms against
  * the library path's 1.39 ms at the benchmark's shape (524288 rows, 3 x 512 -> 512).
@@ -104,7 +104,7 @@ typedef struct HstuOutputArgs {
                                   GEMM's scratch; concatenating path: y (and SiLU(u)) */
     int64_t workspace_bytes;
     int32_t path;              /* 1 = library path (norm-mul kernel + hipBLASLt); 2 = concatenating path (norm-mul kernel
-                                  + hand-written GEMM over the blocks where they are): needs d_out = 512 and heads *
+                                  + hand-written GEMM over the blocks where they are): needs d_out a multiple of 256 and heads *
                                   linear_dim a multiple of 64 (and, with group norm, no SiLU on a copied u), else status
                                   -6; 0 = the concatenating path where it applies and rows >= 32768, else the library */
 } HstuOutputArgs;

@@ -236,6 +236,22 @@ def test_compute_output_concat_gemm_on_views_of_wider_buffers(pkg, dev, N):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("D", [256, 768, 1024])
+def test_compute_output_concat_gemm_other_widths(pkg, dev, D):
+    """d_model = 256, 768, 1024: one, three and four column blocks per row block."""
+    print(f"[case] concat-gemm output d_model={D}", flush=True)
+    N, H, ld = 2000, 2, 64
+    attn, u, x, nw, nb, w = _inputs(500 + D, N, H, ld, D, 3, False, torch.bfloat16)
+    args = (attn.to(dev), u.to(dev), x.to(dev), nw.to(dev), nb.to(dev), 1e-6, w.to(dev), H, ld, 0.0, False, True, True, "silu", False, False)
+    got = pkg.hstu_compute_output(*args, path=2)
+    lib = pkg.hstu_compute_output(*args, path=1)
+    torch.cuda.synchronize()
+    kw = dict(concat_u=True, concat_x=True, mul_u_activation_type="silu")
+    _close(got, O.compute_output(attn, u, x, nw, nb, w, 1e-6, **kw), "other widths: out vs fp32 oracle")
+    _close(got, lib.float().cpu(), "other widths: out vs library path")
+
+
+@pytest.mark.gpu
 def test_compute_output_at_the_benchmark_size(pkg, dev):
     """524288 rows, 3 x 512 -> 512 (the size of `bench.py --workload output`): the automatic choice is the concatenating
     GEMM and it agrees with the library path everywhere; a zero weight returns the residual bit for bit (every row block
