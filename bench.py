@@ -218,7 +218,30 @@ def run_linear(name, args, pkg, torch):
         return (torch.randn(shape, device=dev, generator=g) * scale + shift).to(torch.bfloat16)
 
     x = rnd(L, d_model, scale=1.5, shift=0.3)
-    if name in ("uqvk", "layernorm"):
+    if name == "layer":
+        # one STU layer forward on the headline batch (64 sequences of 8192): hstu_preprocess_and_attention, then
+        # hstu_compute_output on its u and attention output -- the three steps of this library back to back
+        from generative_recommenders_amd import workloads
+
+        wl = workloads.make_workload("headline")
+        offsets = torch.arange(0, L + 1, wl.max_seq_len, dtype=torch.int64, device=dev)
+        nw, nb = rnd(d_model, scale=0.1, shift=1.0), rnd(d_model, scale=0.1)
+        w, b = rnd(d_model, n_out, scale=1.0 / d_model**0.5), rnd(n_out, scale=0.1)
+        onw, onb = rnd(H * D, scale=0.1, shift=1.0), rnd(H * D, scale=0.1)
+        ow = rnd(3 * H * D, d_model, scale=1.0 / (3 * H * D) ** 0.5)
+
+        def step():
+            u, attn, _, _ = hstu_compute.hstu_preprocess_and_attention(
+                x, nw, nb, 1e-6, H, D, D, w, b, wl.max_seq_len, offsets, wl.alpha, True, None, 0, 0, False, False, True)
+            return hstu_compute.hstu_compute_output(attn, u, x, onw, onb, 1e-6, ow, H, D, 0.0, False, True, True, "none", False, False)
+
+        cpu = None
+        attn_flops = workloads.algorithmic_flops(wl)
+        flops = 2.0 * L * d_model * n_out + attn_flops + 2.0 * L * 3 * H * D * d_model
+        nbytes = 2.0 * (L * d_model * 3 + d_model * n_out + 3 * H * D * d_model)  # x in (twice: the residual), out
+        kernel = "hstu_uqvk_fused_kernel + hstu_fwd_pp_kernel + hstu_norm_mul_kernel + hstu_output_gemm_kernel"
+        metric = "STU layer fwd TFLOP/s (uqvk, attention, output; 64 x 8192 tokens, d_model 512, H4 d128)"
+    elif name in ("uqvk", "layernorm"):
         nw, nb = rnd(d_model, scale=0.1, shift=1.0), rnd(d_model, scale=0.1)
         w, b = rnd(d_model, n_out, scale=1.0 / d_model**0.5), rnd(n_out, scale=0.1)
         if name == "uqvk":
@@ -270,7 +293,7 @@ def run_linear(name, args, pkg, torch):
             "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
             "data": "synthetic", "config": {"workload": name, "rows": L, "d_model": d_model, "heads": H, "attn_dim": D, "hidden_dim": D},
             "roofline": roof}
-    if not args.no_cpu:
+    if not args.no_cpu and cpu is not None:
         torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))))
         rows = 32768
         reps, t_used = 0, 0.0
@@ -422,7 +445,7 @@ def main():
     from generative_recommenders_amd import workloads
 
     jagged = args.workload in ("kvcat", "kvtail")
-    producer = args.workload in ("uqvk", "layernorm", "output", "normmul")
+    producer = args.workload in ("uqvk", "layernorm", "output", "normmul", "layer")
     backward = args.workload in ("bwd", "bwd_cfg3")
     wl = None if jagged or producer or backward else workloads.make_workload(args.workload)
     if wl is not None and wl.dtype == "fp32":

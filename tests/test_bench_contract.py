@@ -58,7 +58,7 @@ def test_headline_line_has_the_agreed_shape():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("workload,bound", [("cfg2", "hbm"), ("kvcat", "hbm"), ("normmul", "hbm"), ("bwd_cfg3", "mfma")])
+@pytest.mark.parametrize("workload,bound", [("cfg2", "hbm"), ("kvcat", "hbm"), ("normmul", "hbm"), ("bwd_cfg3", "mfma"), ("layer", "mfma")])
 def test_other_workloads_print_one_line(workload, bound):
     import torch
 
