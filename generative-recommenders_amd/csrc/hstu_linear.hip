@@ -278,9 +278,9 @@ size_t output_fused_workspace(const HstuOutputArgs* a) {
     return ((size_t)a->rows * d * 2 * (output_fused_u_made(a) ? 2 : 1) + 255) & ~(size_t)255;
 }
 
-template <class TT>
+template <class TT, bool BIAS>
 int launch_output_gemm_t(const hstu::OutputGemmParams& p, hipStream_t stream) {
-    auto kern = hstu::hstu_output_gemm_kernel<TT>;
+    auto kern = hstu::hstu_output_gemm_kernel<TT, BIAS>;
     static bool attr_done = false;
     if (!attr_done) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, hstu::kOutLds);
@@ -320,7 +320,8 @@ int launch_output_fused(const HstuOutputArgs* a, hipStream_t stream) {
     for (int i = n; i < 3; ++i) p.src[i] = p.src[0], p.src_rs[i] = p.src_rs[0];
     p.nsrc = n, p.d = d;
     p.x = (const char*)a->x, p.x_rs = a->x_row_stride, p.w = (const char*)a->output_weight, p.out = (char*)a->out, p.rows = a->rows, p.n = a->d_out;
-    return a->dtype == 0 ? launch_output_gemm_t<hstu::Bf16>(p, stream) : launch_output_gemm_t<hstu::Fp16>(p, stream);
+    p.bias = nullptr, p.n_silu = 0;
+    return a->dtype == 0 ? launch_output_gemm_t<hstu::Bf16, false>(p, stream) : launch_output_gemm_t<hstu::Fp16, false>(p, stream);
 }
 
 int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hipStream_t stream) {
@@ -607,7 +608,7 @@ const char* hstu_linear_last_error(void) { return g_last_error; }
 
 size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* a) {
     if (!a || a->rows <= 0 || a->d_model <= 0) return 0;
-    if (a->path != 1 && a->heads > 0 && a->attn_dim > 0 && a->hidden_dim > 0 && uqvk_fused_shape(a)) return 0;
+    if (a->path != 1 && a->path != 3 && a->heads > 0 && a->attn_dim > 0 && a->hidden_dim > 0 && uqvk_fused_shape(a)) return 0;
     return normed_bytes(a) + kGemmScratch;
 }
 
@@ -622,15 +623,25 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
     if (!a) return -1;
     if (a->rows < 0 || a->heads <= 0 || a->attn_dim <= 0 || a->hidden_dim <= 0 || a->d_model <= 0) return -5;
     if (a->rows == 0) return 0;
-    if (a->path < 0 || a->path > 2) return -5;
+    if (a->path < 0 || a->path > 3) return -5;
     if (!a->uvqk_weight || !a->uvqk_bias || !a->uvqk) return -1;
     if (a->rows > 0x7fffffffLL) return -5;
     hipStream_t stream = (hipStream_t)stream_;
     const int n_u = a->hidden_dim * a->heads;
     const int n_out = (2 * a->hidden_dim + 2 * a->attn_dim) * a->heads;
     if ((n_u & 7) != 0 || (n_out & 7) != 0) return -4;  // column blocks start on 16-byte boundaries
-    const bool fused = a->path != 1 && uqvk_fused_shape(a);
+    const bool fused = a->path != 1 && a->path != 3 && uqvk_fused_shape(a);
     if (a->path == 2 && !fused) return -6;
+    // the layer-norm kernel + the hand-written GEMM of the output projection in its bias / SiLU form, on request only
+    // (path 3): with 8 column blocks per row block and a depth of 16 .. 32 tiles it is slower than the library path
+    // (2.23 against 1.72 ms at d_model 512, 3.15 against 2.42 ms at 1024; 524288 rows, 2048 columns)
+    const bool gemm_shape = (a->d_model & 63) == 0 && a->d_model >= 64 && a->d_model <= 4096 && n_out % hstu::kOutWgCols == 0 &&
+                            n_u % hstu::kOutWgCols == 0 && n_out <= 8192 && (a->dtype == 0 || a->dtype == 1);
+    if (a->path == 3 && !gemm_shape) {
+        snprintf(g_last_error, sizeof(g_last_error), "path 3 takes d_model a multiple of 64 and hidden_dim * heads, n_out multiples of 256");
+        return -6;
+    }
+    const bool hand_gemm = a->path == 3;
     if (fused) {
         if (!a->x || !a->norm_weight || !a->norm_bias) return -1;
         if (a->x_row_stride < a->d_model || (a->x_row_stride & 7) != 0) return -5;
@@ -651,6 +662,15 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
     int rc = launch_layer_norm(a->x, a->x_row_stride, a->norm_weight, a->norm_bias, a->norm_eps, normed, a->d_model, a->rows,
                                a->d_model, a->dtype, stream);
     if (rc != 0) return rc;
+    if (hand_gemm) {
+        if ((((uintptr_t)a->uvqk_weight | (uintptr_t)a->uvqk_bias | (uintptr_t)a->uvqk) & 15) != 0) return -4;
+        hstu::OutputGemmParams p;
+        for (int i = 0; i < 3; ++i) p.src[i] = (const char*)normed, p.src_rs[i] = a->d_model;
+        p.nsrc = 1, p.d = a->d_model, p.x = nullptr, p.x_rs = 0;
+        p.w = (const char*)a->uvqk_weight, p.out = (char*)a->uvqk, p.rows = a->rows, p.n = n_out;
+        p.bias = (const char*)a->uvqk_bias, p.n_silu = n_u;
+        return a->dtype == 0 ? launch_output_gemm_t<hstu::Bf16, true>(p, stream) : launch_output_gemm_t<hstu::Fp16, true>(p, stream);
+    }
     // u columns with SiLU in the epilogue, then v | q | k with the bias only
     const char* w = (const char*)a->uvqk_weight;
     const char* b = (const char*)a->uvqk_bias;

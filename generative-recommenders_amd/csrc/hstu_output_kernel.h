@@ -42,6 +42,8 @@ struct OutputGemmParams {
     char* out;           // [rows, n] dense
     int64_t rows;
     int n;               // output columns: a multiple of 256
+    const char* bias;    // BIAS form: [n], added to every row; x is not read
+    int n_silu;          // BIAS form: the first n_silu columns (a multiple of 256) go through SiLU
 };
 
 constexpr int kOutWaves = 4, kOutRows = 256, kOutWgCols = 256, kOutTileK = 32;
@@ -65,7 +67,9 @@ __device__ __forceinline__ void out_step_barrier() {
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
 
-template <class TT>
+// BIAS = false: out = x + rows @ W (the output projection).  BIAS = true: out = act(rows @ W + bias), act = SiLU on the
+// first n_silu columns and nothing on the rest (the q/k/v producer's product for widths its own kernel does not take).
+template <class TT, bool BIAS>
 __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(const OutputGemmParams p) {
     typedef typename TT::vec8 vec8;
     typedef typename TT::elem elem;
@@ -165,13 +169,24 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
             baddr[half][ks] = row * 128 + (((half * 4 + ks * 2 + g) ^ ((row >> 1) & 7)) * 16);
         }
 
+    // accumulator element (dt, 4 r4 + i) of a lane is column dt*32 + r4*8 + g*4 + i of the wave's 128, for its row l32
     f32x16_t acc[4][4];
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int r4 = 0; r4 < 4; ++r4) {
+            float init[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (BIAS) {  // the bias is where the sums start
+                typedef __attribute__((ext_vector_type(4))) elem elem4;
+                const elem4 b4 = *(const elem4*)(p.bias + (colblk * kOutWgCols + cw * 128 + dt * 32 + r4 * 8 + g * 4) * 2);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[rb][dt][r] = 0.f;
+                for (int i = 0; i < 4; ++i) init[i] = (float)b4[i];
+            }
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[rb][dt][r4 * 4 + i] = init[i];
+        }
 
     // The operands of the step in flight and of the one after.  A step is 16 MFMAs with one memory instruction behind
     // each: with one wave per SIMD an LDS read or a copy that is issued in a burst holds up the MFMA behind it, while
@@ -249,19 +264,23 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
     const int chunk = lane & 7, rsub = lane >> 3;  // 8 lanes cover one row's 64 columns, 8 rows per instruction
     const int col0 = colblk * kOutWgCols + cw * 128 + chunk * 8;
     vec8 xr[4][2][4];  // the residual of everything this lane stores, requested at once (rows past the end: the last row)
+    if constexpr (!BIAS) {
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb)
+        for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
+            for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                int64_t r = row0 + rh * 128 + rb * 32 + i * 8 + rsub;
-                r = r < p.rows ? r : p.rows - 1;
-                xr[rb][hf][i] = *(const vec8*)(p.x + (r * p.x_rs + col0 + hf * 64) * 2);
-            }
+                for (int i = 0; i < 4; ++i) {
+                    int64_t r = row0 + rh * 128 + rb * 32 + i * 8 + rsub;
+                    r = r < p.rows ? r : p.rows - 1;
+                    xr[rb][hf][i] = *(const vec8*)(p.x + (r * p.x_rs + col0 + hf * 64) * 2);
+                }
+    }
     // the copies that are still on their way into the rings (repeats of the last tiles) have to land before the staging
     // areas take their place; the 32 loads of the residual behind them need not
-    asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (BIAS) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    const bool silu = BIAS && colblk * kOutWgCols < p.n_silu;
     char* stage = smem + wave * 32 * kOutStageRow;
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
@@ -286,8 +305,14 @@ __global__ __launch_bounds__(kOutWaves * 64, 1) void hstu_output_gemm_kernel(con
                     vec8 ov;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        ov[j] = (elem)(lo[j] + (float)xr[rb][hf][i][j]);
-                        ov[4 + j] = (elem)(hi[j] + (float)xr[rb][hf][i][4 + j]);
+                        if constexpr (BIAS) {
+                            const float a0 = lo[j], a1 = hi[j];
+                            ov[j] = (elem)(silu ? a0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a0)) : a0);
+                            ov[4 + j] = (elem)(silu ? a1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a1)) : a1);
+                        } else {
+                            ov[j] = (elem)(lo[j] + (float)xr[rb][hf][i][j]);
+                            ov[4 + j] = (elem)(hi[j] + (float)xr[rb][hf][i][4 + j]);
+                        }
                     }
                     *(vec8*)(p.out + (r * p.n + col0 + hf * 64) * 2) = ov;
                 }

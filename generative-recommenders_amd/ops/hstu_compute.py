@@ -258,8 +258,10 @@ def hstu_compute_uqvk(
     path: int = 0,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Returns ``(u, q, k, v)``: ``u [L, hidden*H]`` already through SiLU, ``q, k [L, H, attn]``, ``v [L, H, hidden]``,
-    all views of one buffer.  ``path``: 0 = the fused kernel where the shape allows, else layer-norm kernel +
-    hipBLASLt; 1 / 2 force one or the other."""
+    all views of one buffer.  ``path``: 0 = the fused kernel where the shape allows, else the layer-norm kernel +
+    hipBLASLt; 1 = layer-norm kernel + hipBLASLt; 2 = the fused kernel; 3 = layer-norm kernel + hand-written GEMM
+    (d_model a multiple of 64, hidden * H and the output width multiples of 256; slower than 1 at the sizes measured);
+    2 and 3 raise ``NotImplementedError`` where they do not apply."""
     torch._assert(x.dim() == 2, "x must be 2-D")
     n_out = (2 * hidden_dim + 2 * attn_dim) * num_heads
     torch._assert(uvqk_weight.shape == (x.shape[1], n_out), "uvqk_weight must be [d_model, (2*hidden + 2*attn) * heads]")

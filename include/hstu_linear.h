@@ -50,7 +50,11 @@ typedef struct HstuUqvkArgs {
     int32_t path;              /* 0 = automatic: the fused kernel (layer norm, product, bias, SiLU in one pass, the
                                   normalised rows held in registers) when d_model is 128, 256, 384 or 512 and
                                   hidden_dim * heads and n_out are multiples of 128, else the library path;
-                                  1 = library path (layer-norm kernel + hipBLASLt); 2 = fused kernel or status -6 */
+                                  1 = library path (layer-norm kernel + hipBLASLt); 2 = fused kernel or status -6;
+                                  3 = layer-norm kernel + the hand-written GEMM kernel of the output projection with the
+                                  bias as the start of the sums and SiLU(u) in its epilogue (d_model a multiple of 64,
+                                  hidden_dim * heads and n_out multiples of 256, else status -6): never the automatic
+                                  choice, it is the slowest of the three at the widths measured */
 } HstuUqvkArgs;
 
 size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* args);

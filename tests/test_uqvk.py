@@ -179,6 +179,26 @@ def test_compute_uqvk(pkg, dev, L, d_model, H, attn, hidden, dtype, path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize(
+    "L,d_model,H,attn,hidden",
+    [(700, 1024, 4, 128, 128), (1, 64, 2, 128, 128), (300, 512, 4, 128, 128), (5000, 768, 2, 128, 128), (1025, 1024, 8, 64, 64)],
+)
+def test_compute_uqvk_hand_written_gemm(pkg, dev, L, d_model, H, attn, hidden, dtype):
+    """``path=3``: the layer-norm kernel, then the GEMM kernel of the output projection in its bias / SiLU form (the bias
+    as the start of the sums, SiLU on the u columns in the epilogue), on request only.  Same bar as the other paths."""
+    print(f"[case] uqvk gemm {L} {d_model} {H} {attn} {hidden} {dtype}", flush=True)
+    x, nw, nb, w, b = _inputs(L + d_model + 3, L, d_model, H, attn, hidden, dtype)
+    dv = [t.to(dev) for t in (x, nw, nb, w, b)]
+    got = pkg.hstu_compute_uqvk(dv[0], dv[1], dv[2], 1e-6, H, attn, hidden, dv[3], dv[4], path=3)
+    lib = pkg.hstu_compute_uqvk(dv[0], dv[1], dv[2], 1e-6, H, attn, hidden, dv[3], dv[4], path=1)
+    torch.cuda.synchronize()
+    for name, g_, l_, ref in zip("uqkv", got, lib, U.compute_uqvk(x, nw, nb, 1e-6, H, attn, hidden, w, b)):
+        _close(g_, ref, name + " vs fp32 oracle")
+        _close(g_, l_.float().cpu(), name + " vs library path")
+
+
+@pytest.mark.gpu
 def test_uqvk_with_a_total_length_that_changes_from_batch_to_batch(pkg, dev):
     """The hipBLASLt path keeps one plan per size class of the row count, not per row count: lengths of one class
     (1100, 1101, 1279), of others (640, 5000), and the first again, each against the oracle."""
