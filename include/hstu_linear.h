@@ -81,7 +81,7 @@ int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight
  * (one wave per row, HBM-bound) that writes `joined` in the inputs' type; the product with the residual as the GEMM's
  * C operand runs on hipBLASLt.  Concatenating path (d_out a multiple of 256): the same norm-multiply kernel writes y alone (and
  * SiLU(u) where that is a block of `joined`), and a hand-written GEMM kernel reads the blocks of `joined` where they
- * are -- u and attn in the caller's tensors, y in the workspace -- so that `joined` is never written: 1.17 ms against
+ * are -- u and attn in the caller's tensors, y in the workspace -- so that `joined` is never written: 1.15 ms against
  * the library path's 1.39 ms at the benchmark's shape (524288 rows, 3 x 512 -> 512).
  */
 enum { HSTU_MUL_U_NONE = 0, HSTU_MUL_U_SIGMOID = 1, HSTU_MUL_U_SILU = 2 };
