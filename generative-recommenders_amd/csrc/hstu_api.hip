@@ -10,6 +10,7 @@
 
 #include "hstu_fwd_kernel.h"
 #include "hstu_fwd_pp_kernel.h"
+#include "hstu_fwd_stream_kernel.h"
 #include "hstu_jagged_kernels.h"
 
 // Scratch area of hstu_hip_mha_fwd_noalloc: what the caller's `workspace` is to hstu_hip_mha_fwd (work-item counters,
@@ -97,6 +98,7 @@ const TileConfig kConfigs[] = {
     {"m128n64w4", 1, 4, 64},
     {"m256n64w8pp", 1, 8, 64},
     {"m128n64w4pl", 1, 4, 64},
+    {"m256n64w8st", 1, 8, 64},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -127,8 +129,12 @@ int launch(const hstu::FwdParams& p, hipStream_t stream) {
 
 template <class TT, int DQK, int DV, int BN, int NG>
 int launch_pp(const hstu::FwdParams& p, int grid_per_xcd, int64_t total_q, hipStream_t stream) {
-    auto kern = hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN, NG>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid_per_xcd * 8), dim3(NG * 256), 0, stream, p);  // LDS is a static array
+    if constexpr (NG == 0) {  // the streaming form of the 8-wave kernel
+        hipLaunchKernelGGL((hstu::hstu_fwd_stream_kernel<TT, DQK, DV, BN>), dim3((unsigned)grid_per_xcd * 8), dim3(512), 0, stream, p);
+    } else {
+        hipLaunchKernelGGL((hstu::hstu_fwd_pp_kernel<TT, DQK, DV, BN, NG>), dim3((unsigned)grid_per_xcd * 8), dim3(NG * 256), 0, stream,
+                           p);  // LDS is a static array
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         set_last_error("kernel launch", e);
@@ -139,7 +145,7 @@ int launch_pp(const hstu::FwdParams& p, int grid_per_xcd, int64_t total_q, hipSt
         const long long blocks = (threads + 255) / 256;
         if (blocks > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
         hipLaunchKernelGGL(hstu::hstu_reduce_splits_kernel<typename TT::out_elem>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                           p, total_q, DV, NG * 128);
+                           p, total_q, DV, NG == 1 ? 128 : 256);
         e = hipGetLastError();
         if (e != hipSuccess) {
             set_last_error("reduce kernel launch", e);
@@ -153,6 +159,7 @@ template <class TT, int D>
 int launch_cfg(const hstu::FwdParams& p, int cfg, int grid_per_xcd, int64_t total_q, hipStream_t stream) {
     if (cfg == 2) return launch_pp<TT, D, D, 64, 2>(p, grid_per_xcd, total_q, stream);
     if (cfg == 3) return launch_pp<TT, D, D, 64, 1>(p, grid_per_xcd, total_q, stream);
+    if (cfg == 4) return launch_pp<TT, D, D, 64, 0>(p, grid_per_xcd, total_q, stream);
     return launch<TT, D, D, 1, 4, 64, 2>(p, stream);
 }
 
@@ -240,7 +247,7 @@ Plan make_plan(const HstuFwdArgs* a) {
     if (a->sort_by_length && a->batch >= 2 && a->batch <= kMaxSortBatch) pl.order_bytes = (size_t)a->batch * sizeof(int);
     if (pl.cfg < 2 || a->batch <= 0) return pl;
     pl.queue_bytes = 8 * 64 + 64;  // one counter per XCD, 64 bytes apart, then the 8 list lengths
-    const int bm = pl.cfg == 2 ? 256 : 128;
+    const int bm = (pl.cfg == 2 || pl.cfg == 4) ? 256 : 128;
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long blocks = (long long)a->batch * a->heads * ((rows_per_pair + bm - 1) / bm);
     const int max_tiles = (a->max_seq_len + kTileRows - 1) / kTileRows;
@@ -251,7 +258,7 @@ Plan make_plan(const HstuFwdArgs* a) {
         // Delta mode has few query rows per sequence: with a small batch the row blocks alone do not fill the
         // 256 CUs.  Cut the kv range so that the chip is just filled (more runs than that only add partial-sum
         // traffic: with every CU busy the clock drops and the time per tile rises), in runs of at least 16 tiles.
-        const long long resident = pl.cfg == 2 ? 256 : 512;  // workgroups the chip holds at once
+        const long long resident = (pl.cfg == 2 || pl.cfg == 4) ? 256 : 512;  // workgroups the chip holds at once
         long long want = resident / blocks;
         if (want > max_tiles / 16) want = max_tiles / 16;
         if (want > kMaxSplits) want = kMaxSplits;
@@ -535,7 +542,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     const int cfg = plan.cfg;
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long num_pairs = (long long)a->batch * a->heads;
-    const int bm = cfg == 2 ? 256 : 128;
+    const int bm = (cfg == 2 || cfg == 4) ? 256 : 128;
     p.num_mb = (rows_per_pair + bm - 1) / bm;
     const long long pairs_per_xcd = (num_pairs + 7) / 8;
     const long long slots = pairs_per_xcd * p.num_mb * plan.splits;
@@ -543,7 +550,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     if (slots * 8 > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     p.pairs_per_xcd = (int)pairs_per_xcd;
     p.slots_per_xcd = (int)slots;
-    long long resident = (long long)current_device_cus() * (cfg == 2 ? 1 : 2) / 8;
+    long long resident = (long long)current_device_cus() * ((cfg == 2 || cfg == 4) ? 1 : 2) / 8;
     if (resident < 1) resident = 1;
     const int grid_per_xcd = (int)(slots < resident ? slots : resident);
     if (cfg < 2 || slots <= grid_per_xcd) queue = nullptr;  // every workgroup has exactly one item

@@ -96,6 +96,14 @@ struct FwdParams {
 // `out_elem` = type of the output tensor; PRESCALE_Q: multiply Q by c1 when it is loaded (otherwise c1 is
 // applied to the accumulator); `silu` maps one accumulator value to the P value that is rounded and
 // packed by `pack8`, leaving a constant factor to the output scale.
+// %4 .. %7 <- t / (1 + 2^t) for the four values a .. d, side by side; operands %4 .. %7 of the enclosing asm are scratch
+// registers, and the two packed results go to p and q
+#define HSTU_SILU4(a, b, c, d, p, q)                                                                                   \
+    "v_exp_f32 %4, " a "\n\tv_exp_f32 %5, " b "\n\tv_exp_f32 %6, " c "\n\tv_exp_f32 %7, " d "\n\t"                     \
+    "v_add_f32 %4, 1.0, %4\n\tv_add_f32 %5, 1.0, %5\n\tv_add_f32 %6, 1.0, %6\n\tv_add_f32 %7, 1.0, %7\n\t"             \
+    "v_rcp_f32 %4, %4\n\tv_rcp_f32 %5, %5\n\tv_rcp_f32 %6, %6\n\tv_rcp_f32 %7, %7\n\t"                                 \
+    "v_mul_f32 %4, " a ", %4\n\tv_mul_f32 %5, " b ", %5\n\tv_mul_f32 %6, " c ", %6\n\tv_mul_f32 %7, " d ", %7\n\t"     \
+    "v_cvt_pk_bf16_f32 " p ", %4, %5\n\tv_cvt_pk_bf16_f32 " q ", %6, %7\n\t"
 struct Bf16 {
     static constexpr bool PAIRWISE = false;
     typedef bf16x8_t vec8;
@@ -122,6 +130,22 @@ struct Bf16 {
         asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
         return r;
     }
+    // silu + pack8 of eight accumulator values as ONE fixed instruction sequence: four chains side by side, so that no
+    // instruction waits for the one in front of it (a transcendental result is not there for the very next
+    // instruction), in four scratch registers.  Left to the compiler the same work comes out four wide in some copies
+    // of the loop body and strictly serial -- one scratch register, a wait state behind every exp and rcp -- in others,
+    // depending on what else is live around it.
+    static constexpr bool PINNED_SILU = true;
+    static __device__ __forceinline__ vec8 silu_pack8_pinned(const float (&t)[8]) {
+        unsigned p0, p1, p2, p3;
+        float e0, e1, e2, e3;
+        asm volatile(HSTU_SILU4("%8", "%9", "%10", "%11", "%0", "%1") HSTU_SILU4("%12", "%13", "%14", "%15", "%2", "%3")
+                     : "=&v"(p0), "=&v"(p1), "=&v"(p2), "=&v"(p3), "=&v"(e0), "=&v"(e1), "=&v"(e2), "=&v"(e3)
+                     : "v"(t[0]), "v"(t[1]), "v"(t[2]), "v"(t[3]), "v"(t[4]), "v"(t[5]), "v"(t[6]), "v"(t[7]));
+        typedef __attribute__((ext_vector_type(4))) unsigned u4;
+        const u4 r = {p0, p1, p2, p3};
+        return __builtin_bit_cast(vec8, r);
+    }
 };
 // The second instruction of a pair writes the other half of the register the first one wrote, and reads that register
 // to do so; four independent instructions in between cover the latency of the first (the compiler does not see into
@@ -146,6 +170,7 @@ __device__ __forceinline__ void sigmoid_f16_pairs(const h2_t (&t)[4], h2_t (&r)[
 
 struct Fp16 {
     static constexpr bool PAIRWISE = false;
+    static constexpr bool PINNED_SILU = false;
     typedef f16x8_t vec8;
     typedef _Float16 elem;
     typedef _Float16 out_elem;
@@ -184,6 +209,7 @@ struct Fp8 {
     typedef __bf16 out_elem;
     static constexpr int ES = 1;
     static constexpr bool PRESCALE_Q = false;
+    static constexpr bool PINNED_SILU = false;
     static constexpr float PSCALE = 16.0f;
     static __device__ __forceinline__ f32x16_t mfma(vec8 a, vec8 b, f32x16_t c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a, b, c, 0, 0, 0);
@@ -686,6 +712,20 @@ __device__ __forceinline__ void silu_pack(const f32x16_t& s, typename TT::vec8 (
         }
         return;
     }
+    if constexpr (MASK == 0 && TT::PINNED_SILU) {
+        // The hardware does not interlock an MFMA result against a VALU read; the compiler counts the wait states, but
+        // not for reads inside an asm block.  One read it can see (of any register of the accumulator) in front of the
+        // blocks makes it count for them too.
+        asm volatile("" : : "s"(__builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, (float)s[15]))));
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            float t[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) t[j] = s[half * 8 + j];
+            pb[half] = TT::silu_pack8_pinned(t);
+        }
+        return;
+    }
     const int causal_room = row.pos - sp0;  // a key at offset d from sp0 is visible iff d <= causal_room
     unsigned bits = 0;
     if (MASK == 1) bits = row.valid_bits(sp0);
@@ -940,6 +980,29 @@ __global__ __launch_bounds__(256) void hstu_reduce_splits_kernel(const FwdParams
 #pragma unroll
     for (int i = 0; i < 4; ++i) o4[i] = (ELEM)(acc[i] * osc);
     *(elem4*)(p.o + (row * p.o_rs + (int64_t)h * p.o_hs) * 2 + c * 8) = o4;
+}
+
+// The same copy through a buffer descriptor: 16 bytes per lane from descriptor base + soffset (wave-uniform) + voffset
+// (per lane) to LDS at lds_base + 16*lane.  The hardware checks soffset + voffset against the descriptor's size and
+// writes ZEROS to LDS for a lane that lies beyond it (established with a probe on the MI355X: both offsets take part in
+// the check), so a tile that reaches past the end of a sequence needs no clamping: with the size set to the
+// sequence's rows, what follows them (the next sequence, or nothing) is never read.  Issuing a copy costs no vector
+// arithmetic and no 64-bit scalar arithmetic.
+__device__ __forceinline__ i32x4_t make_buffer_rsrc(const char* base_uniform, unsigned bytes) {
+    const uint64_t a = (uint64_t)uniform64((int64_t)(uintptr_t)base_uniform);
+    i32x4_t r;
+    r[0] = (int)(unsigned)a;
+    r[1] = (int)((unsigned)(a >> 32) & 0xFFFFu);  // base[47:32]; stride 0: a raw buffer
+    r[2] = (int)bytes;
+    r[3] = 0x00020000;                            // 32-bit data format, no swizzle
+    return r;
+}
+__device__ __forceinline__ void buffer_load_lds16(i32x4_t rsrc, unsigned voffset, unsigned soffset, const char* lds_base) {
+    const unsigned m0 = (unsigned)(uintptr_t)HSTU_LDS(const char, lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(m0), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory");
 }
 
 // Same copy with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit

@@ -24,48 +24,36 @@
 
 namespace hstu {
 
-// Direct HBM -> LDS copy of one tile, spread over the four "A" waves (copies issued from the "B" waves'
-// matrix phase were measured to stall it; from the A waves they are free); per-lane byte offsets from the
-// tile's first row are precomputed.
+// Direct HBM -> LDS copy of one tile, spread over the four "A" waves (copies issued from the "B" waves' matrix phase
+// were measured to stall it; from the A waves they are free), through a buffer descriptor of the sequence's K (or V)
+// rows for this head: rows past the end of the sequence arrive as zeros.  A lane keeps ONE byte offset per kind of tile:
+// the instructions of a wave lie 256 / CH rows apart, which is a multiple of every swizzle's period, so instruction i
+// differs from instruction 0 only by a number of whole rows, and that goes into the wave-uniform offset together with
+// the tile's first row -- a copy is issued between MFMAs, where every further instruction counts, and costs three
+// scalar instructions besides the copy itself.
 template <int ROWS, int ROWBYTES, bool IS_V, int ES>
 struct TileCopy {
     static constexpr int CH = ROWBYTES / 16;
     static constexpr int NI = ROWS * CH / 64;       // wave-wide copy instructions per tile
     static constexpr int NCW = 4;                   // waves that issue copies
     static constexpr int PER_WAVE = (NI + NCW - 1) / NCW;
-    unsigned off[PER_WAVE];       // for a tile that lies entirely inside the sequence
-    unsigned off_last[PER_WAVE];  // for the sequence's last, partly filled tile: rows past the end re-read the last row
-    static __device__ __forceinline__ unsigned lane_offset(int inst, int lane, int64_t row_stride_bytes, int max_row) {
-        const int p = inst * 64 + lane;
-        int row = p / CH;
-        const int phys = p % CH;
+    static constexpr int STEP = NCW * 64 / CH;      // rows between two instructions of one wave
+    unsigned off0;  // this lane's offset from the tile's first row in the wave's first instruction
+    __device__ __forceinline__ void init(int wave, int lane, unsigned row_stride_bytes) {
+        const int row = (wave * 64 + lane) / CH;
+        const int phys = lane % CH;  // (64 is a multiple of CH)
         const int logical = phys ^ (IS_V ? swz_v<CH, ES>(row) : swz_k<CH>(row));
-        row = row < max_row ? row : max_row;
-        return (unsigned)(row * row_stride_bytes) + logical * 16;
+        off0 = (unsigned)row * row_stride_bytes + logical * 16;
     }
-    __device__ __forceinline__ void init(int wave, int lane, int64_t row_stride_bytes, int n) {
-        const int last_valid = (n - 1) % ROWS;  // last filled row of the sequence's last tile
-#pragma unroll
-        for (int i = 0; i < PER_WAVE; ++i) {
-            off[i] = lane_offset(wave + NCW * i, lane, row_stride_bytes, ROWS);
-            off_last[i] = lane_offset(wave + NCW * i, lane, row_stride_bytes, last_valid);
-        }
-    }
-    // Copy instruction `i` (0 .. PER_WAVE-1) of this wave for the tile starting at row `row0`;
-    // `gbase` points at row 0 of the sequence for this head.
-    __device__ __forceinline__ void issue_one(int i, const char* gbase, int64_t row_stride_bytes, int row0, int n,
-                                              char* lds_tile, int wave) const {
+    // Copy instruction `i` (0 .. PER_WAVE-1) of this wave for the tile starting at row `row0` of the sequence that
+    // `rsrc` describes.
+    __device__ __forceinline__ void issue_one(int i, i32x4_t rsrc, unsigned row_stride_bytes, int row0, char* lds_tile, int wave) const {
         const int inst = wave + NCW * i;
-        if (inst < NI) {
-            const char* tile_base = gbase + (int64_t)row0 * row_stride_bytes;  // wave-uniform
-            const unsigned o = (row0 + ROWS > n) ? off_last[i] : off[i];
-            global_load_lds16_soff(tile_base, o, lds_tile + inst * 1024);
-        }
+        if (inst < NI) buffer_load_lds16(rsrc, off0, (unsigned)(row0 + i * STEP) * row_stride_bytes, lds_tile + inst * 1024);
     }
-    __device__ __forceinline__ void issue(const char* gbase, int64_t row_stride_bytes, int row0, int n, char* lds_tile,
-                                          int wave) const {
+    __device__ __forceinline__ void issue(i32x4_t rsrc, unsigned row_stride_bytes, int row0, char* lds_tile, int wave) const {
 #pragma unroll
-        for (int i = 0; i < PER_WAVE; ++i) issue_one(i, gbase, row_stride_bytes, row0, n, lds_tile, wave);
+        for (int i = 0; i < PER_WAVE; ++i) issue_one(i, rsrc, row_stride_bytes, row0, lds_tile, wave);
     }
 };
 
@@ -172,16 +160,17 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     if (T <= 0) return;  // cannot happen for a row block with rows (each row sees itself); kept for safety
     int t_cur = W.jt_begin;
 
-    const char* kbase = p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * ES;
-    const char* vbase = p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * ES;
-    const int64_t k_rsb = p.k_rs * ES, v_rsb = p.v_rs * ES;
+    // descriptors of the sequence's K and V rows for this head (the host keeps rows * stride below 2^32)
+    const unsigned k_rsb = (unsigned)p.k_rs * ES, v_rsb = (unsigned)p.v_rs * ES;
+    const i32x4_t kbase = make_buffer_rsrc(p.k + (W.seq_start * p.k_rs + (int64_t)W.h * p.k_hs) * ES, (unsigned)n * k_rsb);
+    const i32x4_t vbase = make_buffer_rsrc(p.v + (W.seq_start * p.v_rs + (int64_t)W.h * p.v_hs) * ES, (unsigned)n * v_rsb);
     typedef TileCopy<BN, KROW, false, ES> KCopy;
     typedef TileCopy<BN, VROW, true, ES> VCopy;
     KCopy kcopy;
     VCopy vcopy;
     if (grp == 0) {  // only these waves issue copies
-        kcopy.init(wave, lane_v, k_rsb, n);
-        vcopy.init(wave, lane_v, v_rsb, n);
+        kcopy.init(wave, lane_v, k_rsb);
+        vcopy.init(wave, lane_v, v_rsb);
     }
     constexpr int NPW = KCopy::PER_WAVE + VCopy::PER_WAVE;  // copy instructions per wave and step
     static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
@@ -192,9 +181,9 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     // the prologue, so that the first steps of a workgroup do not each expose a memory latency).
     constexpr int AHEAD = NSLOT - 2;  // 1 or 0
     if (grp == 0) {
-        kcopy.issue(kbase, k_rsb, t_cur * BN, n, smem, wave);
-        vcopy.issue(vbase, v_rsb, t_cur * BN, n, smem + VOFF, wave);
-        kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, n, smem + KTILE, wave);
+        kcopy.issue(kbase, k_rsb, t_cur * BN, smem, wave);
+        vcopy.issue(vbase, v_rsb, t_cur * BN, smem + VOFF, wave);
+        kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
     }
 
     vec8 qreg[KS];
@@ -206,13 +195,13 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     int kaddr[KS];
     int vaddr[2][DT];
     lds_read_offsets<TT, DQK, DV>(kaddr, vaddr, lane_v);
+    // (only vaddr[0] is kept: the second transposing read of an operand lies 8 rows below the first for every lane,
+    // which is an immediate)
 #pragma unroll
-    for (int sec = 0; sec < 2; ++sec)
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            vaddr[sec][dt] += VBIAS;
-            asm volatile("" : "+v"(vaddr[sec][dt]));  // keep the bias in the register, out of the immediates
-        }
+    for (int dt = 0; dt < DT; ++dt) {
+        vaddr[0][dt] += VBIAS;
+        asm volatile("" : "+v"(vaddr[0][dt]));  // keep the bias in the register, out of the immediates
+    }
 
     f32x16_t oacc[DT][1];
 #pragma unroll
@@ -236,9 +225,9 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         const int tv = t_cur + AHEAD < jt_end ? t_cur + AHEAD : jt_end - 1;
         const int tk = t_cur + AHEAD + 1 < jt_end ? t_cur + AHEAD + 1 : jt_end - 1;
         if (j < VCopy::PER_WAVE)
-            vcopy.issue_one(j, vbase, v_rsb, tv * BN, n, smem + VOFF + ((SLOT + AHEAD) % NSLOT) * VTILE, wave);
+            vcopy.issue_one(j, vbase, v_rsb, tv * BN, smem + VOFF + ((SLOT + AHEAD) % NSLOT) * VTILE, wave);
         else
-            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, n, smem + ((SLOT + AHEAD + 1) % NSLOT) * KTILE, wave);
+            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, smem + ((SLOT + AHEAD + 1) % NSLOT) * KTILE, wave);
     };
     // S^T = K Q^T only (first step), K slot chosen at run time.
     auto gemm1_only = [&](int kslot) __attribute__((always_inline)) {
@@ -277,7 +266,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {  // j = 2 sub + tt: the whole 64-row tile in one MFMA
                     const char* vb = vt + ((j >> 1) * 32 + (j & 1) * 16) * VROW;
-                    a[j] = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+                    a[j] = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[0][dt] + 8 * VROW);
                     b[j] = pb[j >> 1][j & 1];
                 }
                 oacc[dt][0] = TT::mfma64(a, b, oacc[dt][0]);
@@ -290,7 +279,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) {
                         const char* vb = vt + (sub * 32 + tt * 16) * VROW;
-                        vec8 a = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+                        vec8 a = read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[0][dt] + 8 * VROW);
                         oacc[dt][0] = TT::mfma(a, pb[sub][tt], oacc[dt][0]);
                     }
         }
@@ -313,7 +302,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
                 for (int j = 0; j < 4; ++j) {
                     if ((m & 1) == 0) {
                         const char* vb = vt + ((j >> 1) * 32 + (j & 1) * 16) * VROW;
-                        a[j] = read_vt_operand<TT>(vb + vaddr[0][o], vb + vaddr[1][o]);
+                        a[j] = read_vt_operand<TT>(vb + vaddr[0][o], vb + vaddr[0][o] + 8 * VROW);
                     } else {
                         a[j] = *HSTU_LDS(const vec8, kt + (o % NS) * 32 * KROW + kaddr[4 * (o / NS) + j]);
                     }
@@ -351,7 +340,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
             if ((k & 1) == 0) {
                 const int sub = o / (2 * DT), tt = (o / DT) % 2, dt = o % DT;
                 const char* vb = vt + (sub * 32 + tt * 16) * VROW;
-                return read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[1][dt]);
+                return read_vt_operand<TT>(vb + vaddr[0][dt], vb + vaddr[0][dt] + 8 * VROW);
             } else {
                 const int ks = o / NS, sub = o % NS;
                 return *HSTU_LDS(const vec8, kt + sub * 32 * KROW + kaddr[ks]);

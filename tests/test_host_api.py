@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol(backend):
     for name in declared:
         assert hasattr(lib, name), name
     assert backend.lib().hstu_hip_version() >= 100
-    assert backend.tile_config_names() == ["m128n64w4", "m256n64w8pp", "m128n64w4pl"]
+    assert backend.tile_config_names() == ["m128n64w4", "m256n64w8pp", "m128n64w4pl", "m256n64w8st"]
 
 
 @pytest.mark.parametrize("struct", ["HstuFwdArgs", "HstuJaggedCopyArgs", "HstuBwdGrads"])
