@@ -485,7 +485,7 @@ def main():
         batch=wl.batch, heads=wl.heads, dqk=wl.dqk, dv=wl.dv, total_q=wl.batch * wl.delta_size if wl.delta_size else wl.total_kv,
         total_kv=wl.total_kv, max_seq_len=wl.max_seq_len, delta_size=wl.delta_size, tile_config=args.tile_config,
         kv_splits=args.kv_splits, sort_by_length=wl.delta_size == 0 and not args.no_sort)
-    roof["kernel"] = {1: "hstu_fwd_kernel", 2: "hstu_fwd_pp_kernel<NG=2>", 3: "hstu_fwd_pp_kernel<NG=1>", 4: "hstu_fwd_stream_kernel"}[cfg]
+    roof["kernel"] = {1: "hstu_fwd_kernel", 2: "hstu_fwd_stream_kernel", 3: "hstu_fwd_pp_kernel<NG=1>"}[cfg]
     roof["kv_splits"] = splits
     roof.update(timing_fields(st))
     roof["algorithmic_flops"] = flops

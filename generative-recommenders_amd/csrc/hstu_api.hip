@@ -98,7 +98,6 @@ const TileConfig kConfigs[] = {
     {"m128n64w4", 1, 4, 64},
     {"m256n64w8pp", 1, 8, 64},
     {"m128n64w4pl", 1, 4, 64},
-    {"m256n64w8st", 1, 8, 64},
 };
 constexpr int kNumConfigs = sizeof(kConfigs) / sizeof(kConfigs[0]);
 
@@ -157,9 +156,8 @@ int launch_pp(const hstu::FwdParams& p, int grid_per_xcd, int64_t total_q, hipSt
 
 template <class TT, int D>
 int launch_cfg(const hstu::FwdParams& p, int cfg, int grid_per_xcd, int64_t total_q, hipStream_t stream) {
-    if (cfg == 2) return launch_pp<TT, D, D, 64, 2>(p, grid_per_xcd, total_q, stream);
-    if (cfg == 3) return launch_pp<TT, D, D, 64, 1>(p, grid_per_xcd, total_q, stream);
-    if (cfg == 4) return launch_pp<TT, D, D, 64, 0>(p, grid_per_xcd, total_q, stream);
+    if (cfg == 2) return launch_pp<TT, D, D, 64, 0>(p, grid_per_xcd, total_q, stream);  // 8 waves, two groups: the streaming kernel
+    if (cfg == 3) return launch_pp<TT, D, D, 64, 1>(p, grid_per_xcd, total_q, stream);  // 4 waves, one group
     return launch<TT, D, D, 1, 4, 64, 2>(p, stream);
 }
 
@@ -211,7 +209,7 @@ struct Plan {
     size_t order_bytes;    // sequence ranking
     size_t counts_bytes;   // runs per row block of a kv-split
     size_t partial_bytes;  // fp32 partial outputs of the runs (256-byte aligned: 256 bytes of slack are added)
-    size_t items_bytes;    // work lists: 8 lists of {b * H + h, row block}
+    size_t items_bytes;    // work lists: 8 lists of 32-byte records (see FwdParams::items)
     size_t cast_bytes;     // fp16 copies of fp32 q, k, v, each 256-byte aligned
     size_t total() const {
         return queue_bytes + order_bytes + counts_bytes + (partial_bytes ? partial_bytes + 256 : 0) + items_bytes + cast_bytes;
@@ -221,6 +219,15 @@ struct Plan {
 constexpr int kMaxSplits = 8;
 constexpr int kTileRows = 64;  // kv rows per tile of every configuration
 
+// The pipelined kernels address the rows of a sequence through buffer descriptors with 32-bit byte offsets: the longest
+// sequence times the largest row stride has to stay below 2^32 bytes.
+bool rows_fit_buffer_offsets(const HstuFwdArgs* a) {
+    const int64_t es = a->dtype == HSTU_FP8_E4M3 ? 1 : 2;
+    int64_t rs = a->q_row_stride > a->k_row_stride ? a->q_row_stride : a->k_row_stride;
+    if (a->v_row_stride > rs) rs = a->v_row_stride;
+    return (int64_t)a->max_seq_len * rs * es < (1LL << 32);
+}
+
 Plan make_plan(const HstuFwdArgs* a) {
     Plan pl = {0, 1, 0, 0, 0, 0, 0, 0, 0};
     // The ping-pong kernel (256-row blocks, one workgroup per CU) wins when the average sequence is long; the
@@ -229,6 +236,7 @@ Plan make_plan(const HstuFwdArgs* a) {
     pl.cfg = a->tile_config;
     const long long avg_tiles = a->batch > 0 ? a->total_kv / a->batch / kTileRows : 0;
     if (a->dqk != a->dv || a->dqk == 16) pl.cfg = 1;  // the only kernel generic in (dqk, dv)
+    if (pl.cfg == 0 && !rows_fit_buffer_offsets(a)) pl.cfg = 1;  // the only kernel with 64-bit row addresses
     if (a->dtype == HSTU_FP32) {
         pl.cfg = 1;  // and the only one with an fp32 store
         pl.cast_bytes = 2 * ((size_t)a->total_q * a->heads * a->dqk + (size_t)a->total_kv * a->heads * (a->dqk + a->dv)) + 4 * 256;
@@ -247,7 +255,7 @@ Plan make_plan(const HstuFwdArgs* a) {
     if (a->sort_by_length && a->batch >= 2 && a->batch <= kMaxSortBatch) pl.order_bytes = (size_t)a->batch * sizeof(int);
     if (pl.cfg < 2 || a->batch <= 0) return pl;
     pl.queue_bytes = 8 * 64 + 64;  // one counter per XCD, 64 bytes apart, then the 8 list lengths
-    const int bm = (pl.cfg == 2 || pl.cfg == 4) ? 256 : 128;
+    const int bm = pl.cfg == 2 ? 256 : 128;
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long blocks = (long long)a->batch * a->heads * ((rows_per_pair + bm - 1) / bm);
     const int max_tiles = (a->max_seq_len + kTileRows - 1) / kTileRows;
@@ -258,18 +266,18 @@ Plan make_plan(const HstuFwdArgs* a) {
         // Delta mode has few query rows per sequence: with a small batch the row blocks alone do not fill the
         // 256 CUs.  Cut the kv range so that the chip is just filled (more runs than that only add partial-sum
         // traffic: with every CU busy the clock drops and the time per tile rises), in runs of at least 16 tiles.
-        const long long resident = (pl.cfg == 2 || pl.cfg == 4) ? 256 : 512;  // workgroups the chip holds at once
+        const long long resident = pl.cfg == 2 ? 256 : 512;  // workgroups the chip holds at once
         long long want = resident / blocks;
         if (want > max_tiles / 16) want = max_tiles / 16;
         if (want > kMaxSplits) want = kMaxSplits;
         if (want >= 2) s = (int)want;
     }
     // Work lists for ragged batches (equal lengths are dealt arithmetically, a kv-split enumerates its runs
-    // arithmetically too): 8 bytes per possible item; beyond 64 MB the arithmetic enumeration stays.
+    // arithmetically too): 32 bytes per possible item; beyond 64 MB the arithmetic enumeration stays.
     const bool uniform = a->delta_size == 0 && a->total_kv == (int64_t)a->batch * a->max_seq_len;
     if (s == 1 && !uniform) {
-        const unsigned long long bytes = (unsigned long long)((a->batch * (long long)a->heads + 7) / 8) * (unsigned long long)((rows_per_pair + bm - 1) / bm) * 64ull;
-        if (bytes <= (64ull << 20)) pl.items_bytes = (size_t)bytes + 8;  // 8: room to align the records
+        const unsigned long long bytes = (unsigned long long)((a->batch * (long long)a->heads + 7) / 8) * (unsigned long long)((rows_per_pair + bm - 1) / bm) * 256ull;
+        if (bytes <= (64ull << 20)) pl.items_bytes = (size_t)bytes + 32;  // 32: room to align the records
     }
     if (s > 1) {
         pl.splits = s;
@@ -278,6 +286,48 @@ Plan make_plan(const HstuFwdArgs* a) {
         pl.partial_bytes = (size_t)s * (size_t)a->total_q * a->heads * a->dv * sizeof(float);
     }
     return pl;
+}
+
+// Constants for fast_div (device side): x / d == (x * magic) >> (32 + shift) for 0 <= x < 2^31; magic 0 means d == 1.
+void fast_div_constants(unsigned d, unsigned* magic, unsigned* shift) {
+    if (d <= 1) {
+        *magic = 0;
+        *shift = 0;
+        return;
+    }
+    unsigned l = 0;
+    while ((1ull << l) < d) ++l;  // ceil(log2 d) >= 1
+    *magic = (unsigned)((1ull << (31 + l)) / d + 1);
+    *shift = l - 1;
+}
+
+void fill_decode_params(hstu::FwdParams& p) {
+    hstu::DecodeParams& d = p.dec;
+    memset(&d, 0, sizeof(d));
+    d.items = p.items;
+    d.nitems = p.nitems;
+    d.order = p.order;
+    d.offsets = p.offsets;
+    d.targets = p.targets;
+    d.items_cap = p.items_cap;
+    d.kv_splits = p.kv_splits;
+    d.kv_chunk = p.kv_chunk;
+    d.c = p.c;
+    d.pairs_per_xcd = p.pairs_per_xcd;
+    d.num_mb = p.num_mb;
+    d.B = p.B;
+    d.H = p.H;
+    d.uniform = p.uniform;
+    d.max_seq_len = p.max_seq_len;
+    d.offsets_i64 = p.offsets_i64;
+    d.targets_i64 = p.targets_i64;
+    d.delta = p.delta;
+    d.w = p.w;
+    d.f = p.f;
+    d.mb_magic = p.mb_magic;
+    d.mb_shift = p.mb_shift;
+    d.h_magic = p.h_magic;
+    d.h_shift = p.h_shift;
 }
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) == 0; }
@@ -398,6 +448,8 @@ int hstu_hip_check_args(const HstuFwdArgs* a) {
         if (d != 32 && d != 64 && d != 128 && !(d == 16 && a->dtype != HSTU_FP8_E4M3)) return HSTU_ERR_BAD_HEAD_DIM;
     // unequal or 16-wide dims and fp32 run on tile config 1 only
     if ((a->dqk != a->dv || a->dqk == 16 || a->dtype == HSTU_FP32) && a->tile_config > 1) return HSTU_ERR_UNSUPPORTED;
+    // ... and so do sequences whose rows span 4 GB or more
+    if (a->tile_config > 1 && !rows_fit_buffer_offsets(a)) return HSTU_ERR_UNSUPPORTED;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;  // nothing to do; pointers may be anything
     if (!a->q || !a->k || !a->v || !a->out || !a->seq_offsets) return HSTU_ERR_NULL_POINTER;
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out)) return HSTU_ERR_MISALIGNED;
@@ -542,7 +594,7 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     const int cfg = plan.cfg;
     const int rows_per_pair = a->delta_size > 0 ? a->delta_size : a->max_seq_len;
     const long long num_pairs = (long long)a->batch * a->heads;
-    const int bm = (cfg == 2 || cfg == 4) ? 256 : 128;
+    const int bm = cfg == 2 ? 256 : 128;
     p.num_mb = (rows_per_pair + bm - 1) / bm;
     const long long pairs_per_xcd = (num_pairs + 7) / 8;
     const long long slots = pairs_per_xcd * p.num_mb * plan.splits;
@@ -550,7 +602,9 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     if (slots * 8 > 0x7fffffffLL) return HSTU_ERR_BAD_SHAPE;
     p.pairs_per_xcd = (int)pairs_per_xcd;
     p.slots_per_xcd = (int)slots;
-    long long resident = (long long)current_device_cus() * ((cfg == 2 || cfg == 4) ? 1 : 2) / 8;
+    fast_div_constants((unsigned)p.num_mb, &p.mb_magic, &p.mb_shift);
+    fast_div_constants((unsigned)p.H, &p.h_magic, &p.h_shift);
+    long long resident = (long long)current_device_cus() * (cfg == 2 ? 1 : 2) / 8;
     if (resident < 1) resident = 1;
     const int grid_per_xcd = (int)(slots < resident ? slots : resident);
     if (cfg < 2 || slots <= grid_per_xcd) queue = nullptr;  // every workgroup has exactly one item
@@ -559,7 +613,13 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     // Equal-length sequences (every one as long as max_seq_len allows): dealing the items with a fixed stride is
     // perfectly balanced and keeps all workgroups of an XCD on the same (sequence, head) pair at the same time,
     // which measures 4-5 % faster than the counter; any other batch needs the counter for balance.
-    if (a->delta_size == 0 && a->total_kv == (int64_t)a->batch * a->max_seq_len) queue = nullptr;
+    if (a->delta_size == 0 && a->total_kv == (int64_t)a->batch * a->max_seq_len) {
+        queue = nullptr;
+        // ... and (the caller's contract: no sequence is longer than max_seq_len) sequence b is rows b * max_seq_len
+        // onwards: the kernels need neither the offsets nor a ranking by length
+        p.uniform = 1;
+        order = nullptr;
+    }
 
     // ahead of the forward kernel: sequence ranking and / or the start value of the work-item counters
     if (order || queue) {
@@ -575,8 +635,8 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
     p.order = order;
     p.queue = queue;
     if (items && queue) {
-        // the lists are 8-byte records behind everything else in the workspace; align them
-        items = (int*)((reinterpret_cast<uintptr_t>(items) + 7) & ~(uintptr_t)7);
+        // the lists are 32-byte records behind everything else in the workspace; align them
+        items = (int*)((reinterpret_cast<uintptr_t>(items) + 31) & ~(uintptr_t)31);
         p.items_cap = (int)slots;
         hipLaunchKernelGGL(hstu::hstu_plan_kernel, dim3(8), dim3(HSTU_PLAN_THREADS), 0, stream, p, bm, 64, queue + 8 * 16, items);
         hipError_t e = hipGetLastError();
@@ -588,6 +648,8 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
         p.nitems = queue + 8 * 16;
     }
 
+    // (after everything above: the block decode_work reads is made of copies)
+    fill_decode_params(p);
     if (a->dtype == HSTU_FP32) return launch_mixed<hstu::Fp16F32>(p, a->dqk, a->dv, stream);
     if (a->dtype == HSTU_BF16) return launch_dim<hstu::Bf16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);
     if (a->dtype == HSTU_FP16) return launch_dim<hstu::Fp16>(p, a->dqk, a->dv, cfg, grid_per_xcd, a->total_q, stream);

@@ -49,6 +49,23 @@ __device__ __forceinline__ int64_t uniform64(int64_t x) {
     return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
+// What decode_work needs of FwdParams, gathered (by the host: fill_decode_params in the API source) into one block of
+// 32 dwords that a wave fetches with two wide scalar loads and one wait.  Read field by field from FwdParams, every
+// field is fetched where it is first needed, behind whatever branch that is, with a wait of its own -- some forty
+// dependent round trips to the scalar cache per decoded item.
+struct DecodeParams {
+    const int* items;
+    const int* nitems;
+    const int* order;
+    const void* offsets;
+    const void* targets;
+    int items_cap, kv_splits, kv_chunk, c, pairs_per_xcd, num_mb, B, H;
+    int uniform, max_seq_len, offsets_i64, targets_i64, delta, w, f, pad0;
+    unsigned mb_magic, mb_shift, h_magic, h_shift;
+    int pad1[2];
+};
+static_assert(sizeof(DecodeParams) == 128, "two loads of 16 dwords");
+
 struct FwdParams {
     const char* q;
     const char* k;
@@ -64,13 +81,17 @@ struct FwdParams {
     int pairs_per_xcd;  // ceil(B*H / 8)
     int slots_per_xcd;  // work items per XCD = pairs_per_xcd * num_mb * kv_splits
     int* queue;         // NULL, or 8 counters 64 bytes apart (one per XCD) handing out work items
-    // NULL, or the work lists built by hstu_plan_kernel: items[xcd * items_cap + i] = {b * H + h, row block},
-    // heaviest class first, nitems[xcd] entries.  Without them item i of an XCD is decoded arithmetically
-    // and may turn out to hold no work (a row block past the end of a short sequence).
+    // NULL, or the work lists built by hstu_plan_kernel: record i of list xcd (8 ints at items[(xcd * items_cap + i) * 8])
+    // = {b, h, row block, n, seq_start (low, high), targets, 0}: everything decode_work would otherwise have to look up
+    // through two dependent loads.  Heaviest class first, nitems[xcd] entries.  Without them item i of an XCD is decoded
+    // arithmetically and may turn out to hold no work (a row block past the end of a short sequence).
     const int* items;
     const int* nitems;
     int items_cap;
     int max_seq_len;
+    int uniform;        // 1: every sequence is exactly max_seq_len long (total_kv == B * max_seq_len under the caller's contract):
+                        // sequence b starts at row b * max_seq_len, and nobody reads the offsets
+    unsigned mb_magic, mb_shift, h_magic, h_shift;  // division by num_mb and by H without a divider (see fast_div)
     int delta;          // 0 = full attention
     int w, c, f;        // max_attn_len, contextual_seq_len, min_full_attn_seq_len
     float c1;           // -alpha * log2(e): Q is multiplied by it when loaded
@@ -90,6 +111,7 @@ struct FwdParams {
     float* partial;
     int64_t partial_stride;  // floats per split = total_q * H * dv
     int* split_counts;
+    alignas(64) DecodeParams dec;  // copies of the fields above that decode_work reads
 };
 
 // Element types.  ES = bytes per element; `vec8` = eight elements = one MFMA operand of a lane;
@@ -398,11 +420,26 @@ __device__ __forceinline__ bool row_block_rows(int nq, int mb, int bm, bool end_
 }
 __device__ __forceinline__ bool row_blocks_end_aligned(const FwdParams& p) { return p.delta == 0 && p.kv_splits <= 1; }
 
-// Decode work item `bid` (the workgroup id in a one-item-per-workgroup launch).  Workgroup ids go round-robin
+// x / d for 0 <= x < 2^31 with constants the host derives from d (fast_div_constants in the API source): with
+// l = ceil(log2 d) and m = floor(2^(31+l) / d) + 1, x / d = (x * m) >> (31 + l); magic 0 stands for d = 1.
+__device__ __forceinline__ int fast_div(int x, unsigned magic, unsigned shift) {
+    return magic ? (int)(__umulhi((unsigned)x, magic) >> shift) : x;
+}
+
+// Decode work item `bid` (the workgroup id in a one-item-per-workgroup launch) of the launch whose FwdParams are the
+// kernel's first argument.  Workgroup ids go round-robin
 // over the 8 XCDs, so ids congruent mod 8 share an L2: all row blocks of one (sequence, head) pair stay on one
 // XCD, heaviest block first.  Returns false if the item holds no work.
 template <int BM, int BN>
-__device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid) {
+__device__ __forceinline__ bool decode_work(Work& w, int bid) {
+    // the block of parameters, straight from the kernel argument segment: FwdParams is the kernels' first argument
+    typedef __attribute__((ext_vector_type(16))) int i32x16_t;
+    struct Two { i32x16_t a, b; };
+    const __attribute__((address_space(4))) char* kernarg = (const __attribute__((address_space(4))) char*)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(kernarg));  // fetched again for every item, not kept in registers across the item loop
+    const __attribute__((address_space(4))) i32x16_t* block = (const __attribute__((address_space(4))) i32x16_t*)(kernarg + __builtin_offsetof(FwdParams, dec));
+    const Two raw = {block[0], block[1]};
+    const DecodeParams p = __builtin_bit_cast(DecodeParams, raw);
     const int xcd = bid & 7;
     int slot = bid >> 3;
     // the splits of one row block are neighbours on one XCD
@@ -416,47 +453,54 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     // the first row block (its contextual rows see every non-target key) is the heaviest of all and runs
     // many times longer than the others, so the first row blocks of all pairs are launched before anything else.
     int pair_local, mb;
-    if (p.items) {
-        // {b * H + h, row block} straight from the list
-        if (slot >= HSTU_CONST(int, p.nitems)[xcd]) return false;
-        const i32x2_t rec = HSTU_CONST(i32x2_t, p.items)[(int64_t)xcd * p.items_cap + slot];
-        const int bh = __builtin_amdgcn_readfirstlane(rec[0]);
-        mb = __builtin_amdgcn_readfirstlane(rec[1]);
-        w.b = bh / p.H;
-        w.h = bh - w.b * p.H;
-        pair_local = 0;
-    } else if (p.c > 0) {
-        if (slot < p.pairs_per_xcd) {
-            pair_local = slot;
-            mb = 0;
-        } else {
-            const int s2 = slot - p.pairs_per_xcd;
-            pair_local = s2 / (p.num_mb - 1);
-            mb = p.num_mb - 1 - (s2 - pair_local * (p.num_mb - 1));
-        }
-    } else {
-        pair_local = slot / p.num_mb;
-        mb = p.num_mb - 1 - (slot - pair_local * p.num_mb);
-    }
-    if (!p.items) {
-    const int pair = pair_local * 8 + xcd;
-    if (pair >= p.B * p.H) return false;
-    const int rseq = pair / p.H;
-    w.h = pair - rseq * p.H;
-    // `order` lists the sequences longest first, so that long sequences start early and are dealt evenly
-    // over the XCDs; it changes the schedule, never the result
-    // The index arrays are read-only for the whole launch and their addresses are wave-uniform: reading
-    // them through the constant address space makes these scalar loads (scalar cache, a fraction of the
-    // latency of a vector load), which matters because three of them are chained at the start of every workgroup.
-    w.b = p.order ? HSTU_CONST(int, p.order)[rseq] : rseq;
-    }
     int64_t seq_start, seq_end;
-    if (p.offsets_i64) {
-        seq_start = HSTU_CONST(int64_t, p.offsets)[w.b];
-        seq_end = HSTU_CONST(int64_t, p.offsets)[w.b + 1];
+    int t = 0;
+    if (p.items) {
+        // everything straight from the list: one load
+        if (slot >= HSTU_CONST(int, p.nitems)[xcd]) return false;
+        typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+        const i32x8_t rec = HSTU_CONST(i32x8_t, p.items)[(int64_t)xcd * p.items_cap + slot];
+        w.b = __builtin_amdgcn_readfirstlane(rec[0]);
+        w.h = __builtin_amdgcn_readfirstlane(rec[1]);
+        mb = __builtin_amdgcn_readfirstlane(rec[2]);
+        seq_start = (int64_t)(((uint64_t)(unsigned)rec[5] << 32) | (unsigned)rec[4]);
+        seq_end = seq_start + rec[3];
+        t = rec[6];
     } else {
-        seq_start = HSTU_CONST(int, p.offsets)[w.b];
-        seq_end = HSTU_CONST(int, p.offsets)[w.b + 1];
+        if (p.c > 0) {
+            if (slot < p.pairs_per_xcd) {
+                pair_local = slot;
+                mb = 0;
+            } else {
+                const int s2 = slot - p.pairs_per_xcd;
+                pair_local = s2 / (p.num_mb - 1);
+                mb = p.num_mb - 1 - (s2 - pair_local * (p.num_mb - 1));
+            }
+        } else {
+            pair_local = fast_div(slot, p.mb_magic, p.mb_shift);
+            mb = p.num_mb - 1 - (slot - pair_local * p.num_mb);
+        }
+        const int pair = pair_local * 8 + xcd;
+        if (pair >= p.B * p.H) return false;
+        const int rseq = fast_div(pair, p.h_magic, p.h_shift);
+        w.h = pair - rseq * p.H;
+        // `order` lists the sequences longest first, so that long sequences start early and are dealt evenly
+        // over the XCDs; it changes the schedule, never the result
+        // The index arrays are read-only for the whole launch and their addresses are wave-uniform: reading
+        // them through the constant address space makes these scalar loads (scalar cache, a fraction of the
+        // latency of a vector load), which matters because they are chained at the start of every item.
+        w.b = p.order ? HSTU_CONST(int, p.order)[rseq] : rseq;
+        if (p.uniform) {
+            seq_start = (int64_t)w.b * p.max_seq_len;
+            seq_end = seq_start + p.max_seq_len;
+        } else if (p.offsets_i64) {
+            seq_start = HSTU_CONST(int64_t, p.offsets)[w.b];
+            seq_end = HSTU_CONST(int64_t, p.offsets)[w.b + 1];
+        } else {
+            seq_start = HSTU_CONST(int, p.offsets)[w.b];
+            seq_end = HSTU_CONST(int, p.offsets)[w.b + 1];
+        }
+        if (p.targets) t = p.targets_i64 ? (int)HSTU_CONST(int64_t, p.targets)[w.b] : HSTU_CONST(int, p.targets)[w.b];
     }
     // Values read from memory are the same for every lane; say so, so that everything derived from
     // them (loop bounds, tile classes, base addresses) lives in scalar registers.
@@ -466,10 +510,8 @@ __device__ __forceinline__ bool decode_work(const FwdParams& p, Work& w, int bid
     w.n = n;
     w.nq = p.delta > 0 ? p.delta : n;
     w.rbase = p.delta > 0 ? n - p.delta : 0;
-    if (n <= 0 || w.rbase < 0 || !row_block_rows(w.nq, mb, BM, row_blocks_end_aligned(p), w.m0, w.m1)) return false;
+    if (n <= 0 || w.rbase < 0 || !row_block_rows(w.nq, mb, BM, (p.delta == 0 && p.kv_splits <= 1), w.m0, w.m1)) return false;
 
-    int t = 0;
-    if (p.targets) t = p.targets_i64 ? (int)HSTU_CONST(int64_t, p.targets)[w.b] : HSTU_CONST(int, p.targets)[w.b];
     t = __builtin_amdgcn_readfirstlane(t);
     SeqMask& M = w.M;
     M.n = n;
@@ -533,30 +575,22 @@ static __global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(con
     const int run = (total + NT - 1) / NT;
     const int k_end = (tid + 1) * run < total ? (tid + 1) * run : total;
     auto walk = [&](bool place) {
-        int cur_pl = -1, bh = 0, n = 0, nq = 0, rbase = 0, u = 0;
+        int cur_pl = -1, b = 0, h = 0, n = 0, nq = 0, rbase = 0, u = 0, t = 0;
+        int64_t seq_start = 0;
         bool live = false;
         SeqMask M;
+        auto put = [&](int pos, int mb) {  // record `pos` of this XCD's list
+            if (pos < p.items_cap) {
+                typedef __attribute__((ext_vector_type(4))) int i32x4;
+                i32x4* rec = (i32x4*)(items + 8 * ((int64_t)xcd * p.items_cap + pos));
+                rec[0] = (i32x4){b, h, mb, n};
+                rec[1] = (i32x4){(int)(unsigned)(uint64_t)seq_start, (int)(unsigned)((uint64_t)seq_start >> 32), t, 0};
+            }
+        };
         for (int k = tid * run; k < k_end; ++k) {
             const int pl = k / num_mb;
             const int mb = num_mb - 1 - (k - pl * num_mb);  // heaviest block of a pair first
-            if (place && k < CACHE) {
-                // second walk: the class is known, only the pair's identity has to be looked up again
-                const int c = cls[k];
-                if (c < 0) continue;
-                if (pl != cur_pl) {
-                    cur_pl = pl;
-                    const int pair = pl * 8 + xcd;
-                    const int rseq = pair / p.H;
-                    bh = (p.order ? p.order[rseq] : rseq) * p.H + (pair - rseq * p.H);
-                }
-                const int pos = cbase[c] + cnt[c][tid];
-                if (pos < p.items_cap) {
-                    items[2 * ((int64_t)xcd * p.items_cap + pos)] = bh;
-                    items[2 * ((int64_t)xcd * p.items_cap + pos) + 1] = mb;
-                }
-                cnt[c][tid] += 1;
-                continue;
-            }
+            if (place && k < CACHE && cls[k] < 0) continue;  // second walk: known not to exist
             if (!place && k < CACHE) cls[k] = -1;
             if (pl != cur_pl) {
                 cur_pl = pl;
@@ -564,15 +598,15 @@ static __global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(con
                 live = pair < p.B * p.H;
                 if (live) {
                     const int rseq = pair / p.H;
-                    const int b = p.order ? p.order[rseq] : rseq;
-                    bh = b * p.H + (pair - rseq * p.H);
-                    const int64_t len = p.offsets_i64 ? ((const int64_t*)p.offsets)[b + 1] - ((const int64_t*)p.offsets)[b]
-                                                      : (int64_t)(((const int*)p.offsets)[b + 1] - ((const int*)p.offsets)[b]);
+                    b = p.order ? p.order[rseq] : rseq;
+                    h = pair - rseq * p.H;
+                    seq_start = p.offsets_i64 ? ((const int64_t*)p.offsets)[b] : (int64_t)((const int*)p.offsets)[b];
+                    const int64_t len = (p.offsets_i64 ? ((const int64_t*)p.offsets)[b + 1] : (int64_t)((const int*)p.offsets)[b + 1]) - seq_start;
                     n = len > p.max_seq_len ? p.max_seq_len : (int)len;
                     nq = p.delta > 0 ? p.delta : n;
                     rbase = p.delta > 0 ? n - p.delta : 0;
                     live = n > 0 && rbase >= 0;
-                    int t = 0;
+                    t = 0;
                     if (p.targets) t = p.targets_i64 ? (int)((const int64_t*)p.targets)[b] : ((const int*)p.targets)[b];
                     M.n = n;
                     M.w = p.w;
@@ -584,22 +618,21 @@ static __global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(con
                     M.idclamp = p.targets ? M.max_id : 0x7fffffff;
                 }
             }
-            int m0, m1;
-            if (!live || !row_block_rows(nq, mb, bm, row_blocks_end_aligned(p), m0, m1)) continue;
-            int jb, je;
-            kv_tile_range(M, u, rbase + m0, rbase + m1 - 1, bn, jb, je);
-            const int tiles = je - jb;
-            if (tiles <= 0) continue;
-            int c = 31 - __builtin_clz((unsigned)tiles);
-            c = c > NC - 1 ? NC - 1 : c;
-            if (!place && k < CACHE) cls[k] = (signed char)c;
-            if (place) {
-                const int pos = cbase[c] + cnt[c][tid];
-                if (pos < p.items_cap) {
-                    items[2 * ((int64_t)xcd * p.items_cap + pos)] = bh;
-                    items[2 * ((int64_t)xcd * p.items_cap + pos) + 1] = mb;
-                }
+            int c;
+            if (place && k < CACHE) {
+                c = cls[k];  // the class is remembered from the first walk
+            } else {
+                int m0, m1;
+                if (!live || !row_block_rows(nq, mb, bm, row_blocks_end_aligned(p), m0, m1)) continue;
+                int jb, je;
+                kv_tile_range(M, u, rbase + m0, rbase + m1 - 1, bn, jb, je);
+                const int tiles = je - jb;
+                if (tiles <= 0) continue;
+                c = 31 - __builtin_clz((unsigned)tiles);
+                c = c > NC - 1 ? NC - 1 : c;
+                if (!place && k < CACHE) cls[k] = (signed char)c;
             }
+            if (place) put(cbase[c] + cnt[c][tid], mb);
             cnt[c][tid] += 1;
         }
     };

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void hstu_fwd_kernel(const FwdParams 
     const int l32 = lane & 31;    // operand row (A) / column (B, C) this lane holds
 
     Work W;
-    if (!decode_work<BM, BN>(p, W, blockIdx.x)) return;
+    if (!decode_work<BM, BN>(W, blockIdx.x)) return;
     const SeqMask& M = W.M;
     const int n = W.n;
     const int nq = W.m1;  // one past the last row of this item: rows from here on are never loaded or stored

@@ -126,7 +126,7 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     asm volatile("" : "+s"(pk));
     const FwdParams& p = *(const FwdParams*)pk;
     Work W;
-    if (!decode_work<BM, BN>(p, W, bid)) return;
+    if (!decode_work<BM, BN>(W, bid)) return;
     const SeqMask& M = W.M;
     const int n = W.n;
     const int nq = W.m1;  // one past the last row of this item: rows from here on are never loaded or stored

@@ -407,7 +407,7 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_stream_kernel(const FwdParams
     auto find_next = [&](const FwdParams& p, Work& W) __attribute__((always_inline)) -> bool {
         for (;;) {
             if (next_bid < 0) return false;
-            if (decode_work<BM, BN>(p, W, next_bid) && W.jt_end > W.jt_begin) return true;
+            if (decode_work<BM, BN>(W, next_bid) && W.jt_end > W.jt_begin) return true;
             if (queue) {
                 if (drawer) publish_next(resolve_ticket(draw_ticket()));
                 __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
@@ -566,11 +566,13 @@ __global__ __launch_bounds__(512, 2) void hstu_fwd_stream_kernel(const FwdParams
             }
             if (rem >= 1) stepA(S1{});
             if (rem >= 2) stepA(S2{});
-            // the Q registers and the K slots are dead: the next item's loads go out ahead of the drain
+            // The K slots are dead: the next item's copies go out ahead of the output.  (The last second product first:
+            // the other group starts its copies of the next Q rows now, and the vector memory path takes one 1 KB copy
+            // per 16 cycles -- this group's 20 per wave would only stand in their way, while it has time to spare.)
             more = find_next(params(), W);
             v0_late = rem == 0;  // the drain reads V slot (T - 1) % 3
-            if (more) prefetch(params(), W, lane_again(), G{});
             gemm2_only(rem);
+            if (more) prefetch(params(), W, lane_again(), G{});
             store_item(params(), more);
         }
     } else {

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol(backend):
     for name in declared:
         assert hasattr(lib, name), name
     assert backend.lib().hstu_hip_version() >= 100
-    assert backend.tile_config_names() == ["m128n64w4", "m256n64w8pp", "m128n64w4pl", "m256n64w8st"]
+    assert backend.tile_config_names() == ["m128n64w4", "m256n64w8pp", "m128n64w4pl"]
 
 
 @pytest.mark.parametrize("struct", ["HstuFwdArgs", "HstuJaggedCopyArgs", "HstuBwdGrads"])
@@ -151,14 +151,14 @@ def test_check_args_status_codes(backend):
     assert chk(dtype=0, k_row_stride=4 * 128 + 8) == 0
     assert chk(workspace=0x1002, workspace_bytes=64) == -4
     # workspace of the persistent kernels (tile configs 2 and 3): 8 work-item counters 64 bytes apart and 8 list
-    # lengths (576 bytes); for batches that are not all of length max_seq_len the work lists (64 bytes per possible
-    # item of one XCD, + 8); for sort_by_length one int per sequence
+    # lengths (576 bytes); for batches that are not all of length max_seq_len the work lists (a 32-byte record per possible
+    # item and XCD, + 32 to align them); for sort_by_length one int per sequence
     need = lambda **o: backend.lib().hstu_hip_workspace_bytes(ctypes.byref(_args(backend, **o)))  # noqa: E731
-    assert need() == 576 + (1 * 1 * 64 + 8)
+    assert need() == 576 + (1 * 1 * 256 + 32)
     assert need(total_q=128, total_kv=128) == 576  # 2 sequences of exactly max_seq_len = 64
     assert need(tile_config=1) == 0
-    assert need(sort_by_length=1, batch=64) == 576 + 256 + (32 * 1 * 64 + 8)
-    assert need(sort_by_length=1, batch=1) == 576 + (1 * 1 * 64 + 8)
+    assert need(sort_by_length=1, batch=64) == 576 + 256 + (32 * 1 * 256 + 32)
+    assert need(sort_by_length=1, batch=1) == 576 + (1 * 1 * 256 + 32)
     assert need(sort_by_length=1, batch=64, tile_config=1) == 256
     for rc in range(-8, 1):
         assert backend.lib().hstu_hip_status_string(rc)
