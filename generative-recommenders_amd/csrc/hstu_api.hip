@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 #include <initializer_list>
+#include <mutex>
 
 #include "hstu_fwd_kernel.h"
 #include "hstu_fwd_pp_kernel.h"
@@ -107,14 +108,18 @@ int launch(const hstu::FwdParams& p, hipStream_t stream) {
     // + 64: with dv = 16 the transposing reads of the unused upper half of the tile reach past the last V row
     constexpr int smem = 2 * BN * (DQK + DV) * TT::ES + 64;
     auto kern = hstu::hstu_fwd_kernel<TT, DQK, DV, QT, NW, BN, OCC>;
-    static bool attr_done = false;  // raising the dynamic LDS limit is idempotent; racing threads set the same value
-    if (!attr_done) {
+    // once per device (the attribute belongs to the device's copy of the kernel); raising the dynamic LDS limit is
+    // idempotent, so racing threads only set the same value twice
+    static bool attr_done[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    if (dev < 0 || !attr_done[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) {
             set_last_error("hipFuncSetAttribute", e);
             return HSTU_ERR_LAUNCH;
         }
-        attr_done = true;
+        if (dev >= 0) attr_done[dev] = true;
     }
     const long long grid = (long long)p.slots_per_xcd * 8;  // one workgroup per work item
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(NW * 64), smem, stream, p);
@@ -384,7 +389,7 @@ extern "C" __attribute__((visibility("hidden"))) int hstu_hip_launch_rank(const 
 
 extern "C" {
 
-int hstu_hip_version(void) { return 100; }
+int hstu_hip_version(void) { return 101; }
 
 const char* hstu_hip_status_string(int status) {
     switch (status) {
@@ -399,6 +404,7 @@ const char* hstu_hip_status_string(int status) {
         case HSTU_ERR_LAUNCH: return "HIP launch failed";
         case HSTU_ERR_BAD_DEVICE: return "current device is not gfx950";
         case HSTU_ERR_SCRATCH_LIMIT: return "the call needs more scratch memory than the library's fixed area holds";
+        case HSTU_ERR_BUSY: return "the library's fixed scratch area is still in use by a call on another stream";
         default: return "unknown status";
     }
 }
@@ -470,8 +476,9 @@ int hstu_hip_check_contract(const HstuFwdArgs* a, int32_t* report, void* stream_
     if (rc != HSTU_OK) return rc;
     if (!report) return HSTU_ERR_NULL_POINTER;
     hipStream_t stream = (hipStream_t)stream_;
-    // a small fill kernel would do as well; this memset is outside anything a caller captures (the check reads back)
-    const int32_t init[4] = {0, 0x7fffffff, 0, 0};
+    // a small fill kernel would do as well; this copy is outside anything a caller captures (the check reads back).
+    // The source outlives the call: an asynchronous copy from pageable memory may read it after this function returns.
+    static const int32_t init[4] = {0, 0x7fffffff, 0, 0};
     hipError_t e = hipMemcpyAsync(report, init, sizeof(init), hipMemcpyHostToDevice, stream);
     if (e != hipSuccess) {
         set_last_error("hipMemcpyAsync", e);
@@ -658,27 +665,41 @@ int hstu_hip_mha_fwd(const HstuFwdArgs* a, void* stream_) {
 
 namespace {
 
-// Device address of `scratch` on the current device (each device holds its own copy of the array at its own address),
-// looked up once per device with that device current; NULL if the lookup fails.
-void* noalloc_scratch_of_current_device() {
-    static void* cache[64];  // racing threads store the same value
+// Per device, set up on the first call with that device current: the device address of `scratch` (each device holds
+// its own copy of the array at its own address) and an event that marks the end of the last call that used the area.
+struct NoallocState {
+    void* scratch = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t last_stream = nullptr;
+    bool in_use = false;  // `done` has been recorded
+};
+std::mutex g_noalloc_mutex;
+
+NoallocState* noalloc_state_of_current_device() {
+    static NoallocState state[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    if (!cache[dev]) {
+    NoallocState& st = state[dev];
+    if (!st.scratch) {
         void* ptr = nullptr;
         hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
         if (e != hipSuccess || !ptr) {
             set_last_error("hipGetSymbolAddress(scratch)", e);
             return nullptr;
         }
-        cache[dev] = ptr;
+        e = hipEventCreateWithFlags(&st.done, hipEventDisableTiming);
+        if (e != hipSuccess) {
+            set_last_error("hipEventCreateWithFlags", e);
+            return nullptr;
+        }
+        st.scratch = ptr;
     }
-    return cache[dev];
+    return &st;
 }
 
 }  // namespace
 
-int hstu_hip_mha_fwd_noalloc(const HstuFwdArgs* a, void* stream) {
+int hstu_hip_mha_fwd_noalloc(const HstuFwdArgs* a, void* stream_) {
     g_last_error[0] = 0;
     int rc = hstu_hip_check_args(a);
     if (rc != HSTU_OK) return rc;
@@ -690,15 +711,30 @@ int hstu_hip_mha_fwd_noalloc(const HstuFwdArgs* a, void* stream) {
                  (size_t)HSTU_NOALLOC_SCRATCH_BYTES);
         return HSTU_ERR_SCRATCH_LIMIT;
     }
-    void* ptr = noalloc_scratch_of_current_device();
-    if (!ptr) return HSTU_ERR_LAUNCH;
+    hipStream_t stream = (hipStream_t)stream_;
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);  // check, launch and record belong together
+    NoallocState* st = noalloc_state_of_current_device();
+    if (!st) return HSTU_ERR_LAUNCH;
+    // A call on another stream while the last one has not finished would race on the area.  (Not under capture: an
+    // event recorded into a graph cannot be queried, and a captured launch runs whenever the graph is replayed.)
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
+    if (!capturing && st->in_use && st->last_stream != stream && hipEventQuery(st->done) == hipErrorNotReady) {
+        snprintf(g_last_error, sizeof(g_last_error), "the scratch area of this device is in use by a call on another stream");
+        return HSTU_ERR_BUSY;
+    }
     HstuFwdArgs b = *a;
-    b.workspace = ptr;  // the device address, never the array's name
+    b.workspace = st->scratch;  // the device address, never the array's name
     b.workspace_bytes = (int64_t)HSTU_NOALLOC_SCRATCH_BYTES;
     // Everything the kernels read from the area is written earlier in the same call (counters and ranking by the prep
     // kernel, work lists by the plan kernel, run counts and partial sums by the forward kernel), so what an earlier
     // call left behind is never looked at and nothing has to be cleared.
-    return hstu_hip_mha_fwd(&b, stream);
+    rc = hstu_hip_mha_fwd(&b, stream_);
+    if (rc == HSTU_OK && !capturing && hipEventRecord(st->done, stream) == hipSuccess) {
+        st->last_stream = stream;
+        st->in_use = true;
+    }
+    return rc;
 }
 
 }  // extern "C"

@@ -132,6 +132,9 @@ extern "C" int hstu_hip_mha_bwd(const HstuFwdArgs* a, const HstuBwdGrads* g, voi
     if (rc != HSTU_OK) return rc;
     if (a->delta_size != 0) return HSTU_ERR_UNSUPPORTED;
     if (a->dtype != HSTU_BF16 && a->dtype != HSTU_FP16) return HSTU_ERR_UNSUPPORTED;
+    // the kernels scale by 1 / max_seq_len: a caller with an attn_scale multiplies dout by attn_scale * max_seq_len
+    // itself (a per-row factor commutes with everything behind it) and calls with attn_scale = NULL
+    if (a->attn_scale) return HSTU_ERR_UNSUPPORTED;
     if (a->total_q == 0 || a->batch == 0) return HSTU_OK;
     if (!g->dout || !g->dq || !g->dk || !g->dv) return HSTU_ERR_NULL_POINTER;
     const uintptr_t ptrs = reinterpret_cast<uintptr_t>(g->dout) | reinterpret_cast<uintptr_t>(g->dq) |

@@ -181,6 +181,7 @@ _STATUS_EXC = {
     -7: RuntimeError,
     -8: RuntimeError,
     -9: RuntimeError,
+    -10: RuntimeError,
 }
 
 

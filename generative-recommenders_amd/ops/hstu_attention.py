@@ -19,6 +19,7 @@ messages and output shapes.  Differences, all explicit:
   they change the schedule, and with a split the fp32 summation order, never the mask or the scaling.
 """
 
+import functools
 from typing import Optional
 
 import torch
@@ -106,6 +107,22 @@ def _require_device(t: torch.Tensor, name: str) -> None:
     torch._assert(t.is_cuda, f"{name} must be CUDA tensor")
 
 
+def _profiled(name: str):
+    """Runs the operator inside a ``torch.profiler.record_function`` range, so that it shows up by name in a trace as the
+    reference's ranges around the same calls do (``modules/stu.py:303,392``)."""
+
+    def decorate(fn):
+        @functools.wraps(fn)
+        def wrapper(*args, **kwargs):
+            with torch.profiler.record_function(name):
+                return fn(*args, **kwargs)
+
+        return wrapper
+
+    return decorate
+
+
+@_profiled("hstu_mha")
 def hstu_mha(
     max_seq_len: int,
     alpha: float,
@@ -206,6 +223,7 @@ def hstu_mha(
     return out
 
 
+@_profiled("delta_hstu_mha")
 def delta_hstu_mha(
     max_seq_len: int,
     alpha: float,

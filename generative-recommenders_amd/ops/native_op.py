@@ -76,6 +76,9 @@ def _forward(
         num_targets = _index_tensor(num_targets, "num_targets")
     if attn_scale is not None:
         _check(attn_scale.numel() in (1, q.shape[0]), "attn_scale: one element, or one per row of q")
+        if torch.is_grad_enabled() and attn_scale.requires_grad:
+            # (as generative_recommenders_amd.hstu_mha does: silently returning no gradient would be worse)
+            raise NotImplementedError("hstu_mha: no gradient is computed for attn_scale; pass it detached")
         attn_scale = attn_scale.detach().to(torch.float32)
         attn_scale = attn_scale.reshape(()) if attn_scale.numel() == 1 else attn_scale.reshape(-1).contiguous()
     out_dtype = torch.bfloat16 if q.dtype == torch.float8_e4m3fn else q.dtype  # flash_common.cpp:596-607
@@ -138,7 +141,8 @@ def _backward(ctx, dout) -> Tuple[Optional[torch.Tensor], ...]:
     max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len = ctx.params
     _check(q.dtype in (torch.float16, torch.bfloat16), "hstu_mha backward: fp16 and bf16 only")
     q, k, v = _kernel_layout(q.detach()), _kernel_layout(k.detach()), _kernel_layout(v.detach())
-    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    # (as the other autograd path: the kernels write every row of every sequence that keeps the caller's contract)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     if q.numel() > 0:
         if attn_scale is not None:
             factor = attn_scale.detach().float() * float(max_seq_len)

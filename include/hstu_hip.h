@@ -42,7 +42,9 @@ enum HstuStatus {
     HSTU_ERR_UNSUPPORTED = -6,    /* legal in the reference but not built here */
     HSTU_ERR_LAUNCH = -7,         /* hipLaunchKernel failed; see hstu_hip_last_error() */
     HSTU_ERR_BAD_DEVICE = -8,     /* the current device is not gfx950 */
-    HSTU_ERR_SCRATCH_LIMIT = -9   /* hstu_hip_mha_fwd_noalloc: the call needs more than HSTU_NOALLOC_SCRATCH_BYTES */
+    HSTU_ERR_SCRATCH_LIMIT = -9,  /* hstu_hip_mha_fwd_noalloc: the call needs more than HSTU_NOALLOC_SCRATCH_BYTES */
+    HSTU_ERR_BUSY = -10           /* hstu_hip_mha_fwd_noalloc: the device's scratch area is still in use by a call that was
+                                     launched on another stream */
 };
 
 /*
@@ -102,7 +104,8 @@ typedef struct HstuFwdArgs {
     int32_t attn_scale_per_row;
 } HstuFwdArgs;
 
-/* Library version, major*10000 + minor*100 + patch. */
+/* Library version, major*10000 + minor*100 + patch.  101: HstuFwdArgs gained attn_scale / attn_scale_per_row at its end
+ * (a caller built against 100 passes a shorter struct and must be rebuilt). */
 int hstu_hip_version(void);
 
 /* Static, human-readable text for a status code. */
@@ -149,9 +152,13 @@ int hstu_hip_check_contract(const HstuFwdArgs* args, int32_t* report, void* stre
  * hstu_hip_workspace_bytes(args) exceeds the area -- FP32 inputs of more than a few million elements (their fp16
  * copies live there), kv-splits of very large delta batches, work lists of more than about 6 million row blocks.
  * All calls on one device share that device's area: two calls that may run at the same time on one device (different
- * streams, or different threads) race on it and must be serialised by the caller; calls on one stream are safe back
- * to back.  Nothing needs clearing between calls (every word a kernel reads was written earlier in the same call).
- * The first call on a device looks the area's address up (hipGetSymbolAddress); make that call outside a capture.
+ * streams) race on it and must be serialised by the caller; calls on one stream are safe back to back.  The library
+ * catches the common form of the mistake without synchronising anything: it records an event behind every call and
+ * returns HSTU_ERR_BUSY (nothing launched) when a call arrives on a DIFFERENT stream while the event of the call before
+ * has not completed.  Under stream capture neither is possible (an event recorded into a graph cannot be queried), so
+ * the check is skipped there and the caller's discipline is all there is.  Nothing needs clearing between calls (every
+ * word a kernel reads was written earlier in the same call).  The first call on a device looks the area's address up
+ * (hipGetSymbolAddress) and creates that event; make that call outside a capture.
  */
 #define HSTU_NOALLOC_SCRATCH_BYTES (48u << 20)
 int hstu_hip_mha_fwd_noalloc(const HstuFwdArgs* args, void* stream);
@@ -185,7 +192,9 @@ const char* hstu_hip_tile_config_name(int id);
  * written; no atomics, so the result is bit-identical from run to run.  The gradients have the layout rules of
  * q / k / v: 16-byte aligned base, row and head strides in elements and multiples of 8, innermost stride 1.
  * `sort_by_length` (a scheduling hint: long sequences first) takes effect when `args->workspace` holds at least
- * 4 * batch bytes.
+ * 4 * batch bytes.  `args->attn_scale` must be NULL (HSTU_ERR_UNSUPPORTED otherwise): the gradients are those of the
+ * 1 / max_seq_len scale; for a forward call that was given an attn_scale, multiply dout row by row by
+ * attn_scale * max_seq_len first (the factor is per query row and commutes with everything behind it).
  *
  * Two ways to form dq.  Without more workspace than that, a second kernel recomputes the scores and dP from the query
  * side (seven matrix products for the five the mathematics needs).  With a 256-byte aligned workspace of at least

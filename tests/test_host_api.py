@@ -160,12 +160,25 @@ def test_check_args_status_codes(backend):
     assert need(sort_by_length=1, batch=64) == 576 + 256 + (32 * 1 * 256 + 32)
     assert need(sort_by_length=1, batch=1) == 576 + (1 * 1 * 256 + 32)
     assert need(sort_by_length=1, batch=64, tile_config=1) == 256
-    for rc in range(-8, 1):
+    for rc in range(-10, 1):
         assert backend.lib().hstu_hip_status_string(rc)
     with pytest.raises(RuntimeError):
         backend.raise_for_status(-3)
     with pytest.raises(ValueError):
         backend.raise_for_status(-5)
+
+
+def test_backward_rejects_attn_scale(backend):
+    """The backward kernels scale by 1 / max_seq_len; a call that carries the forward's attn_scale is refused before
+    anything touches the device (the caller scales dout instead)."""
+    a = _args(backend, attn_scale=0x3000)
+    g = backend.HstuBwdGrads()
+    g.dout = g.dq = g.dk = g.dv = 0x4000
+    for s in ("do", "dq", "dk", "dv"):
+        setattr(g, f"{s}_row_stride", 4 * 128)
+        setattr(g, f"{s}_head_stride", 128)
+    assert backend.lib().hstu_hip_mha_bwd(ctypes.byref(a), ctypes.byref(g), None) == -6
+    assert backend.lib().hstu_hip_version() >= 101  # HstuFwdArgs ends with attn_scale, attn_scale_per_row
 
 
 def test_python_mirror_keeps_reference_assertions(pkg):

@@ -52,6 +52,49 @@ def test_noalloc_entry_point_matches_the_workspace_one(pkg, dev):
             assert torch.equal(a, b), f"delta form, {B} users, kv_splits {splits}"
 
 
+def test_noalloc_entry_point_allocates_nothing_and_refuses_overlap(pkg, dev):
+    """What the entry point is for: after the first call on the device (which looks the area up) a call changes neither
+    the framework's allocated bytes nor the device's free memory, and takes no workspace from the caller.  And the
+    misuse it can detect: a call on another stream while the last one is still running is refused, not raced."""
+    from generative_recommenders_amd.ops import hip_backend
+
+    print("[case] noalloc: memory before / after, then a call on a second stream while the first is running", flush=True)
+    rng = np.random.default_rng(78)
+    lengths = rng.integers(1, 900, size=40)
+    q, k, v, offs, t = [x.to(dev) for x in make_case(int(lengths.sum()), lengths, 2, 128, targets=np.zeros(40, dtype=np.int64))]
+    out = torch.empty((q.shape[0], 2, 128), dtype=q.dtype, device=dev)
+    kw = dict(max_seq_len=900, alpha=0.08, delta_size=0, max_attn_len=0, contextual_seq_len=0, min_full_attn_seq_len=0,
+              sort_by_length=True, noalloc=True, workspace_bytes=0)  # workspace_bytes=0: args.workspace stays NULL
+    hip_backend.mha_fwd(q, k, v, out, offs, t, **kw)
+    torch.cuda.synchronize()
+    before = (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev), torch.cuda.mem_get_info(dev)[0])
+    hip_backend.mha_fwd(q, k, v, out, offs, t, **kw)
+    torch.cuda.synchronize()
+    after = (torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev), torch.cuda.mem_get_info(dev)[0])
+    assert before == after, (before, after)
+
+    # a long call (64 sequences of 4096: about a millisecond) on one stream, then at once a small one on another
+    big = np.full(64, 4096)
+    qb, kb, vb, ob, tb = [x.to(dev) for x in make_case(5, big, 4, 128, targets=np.zeros(64, dtype=np.int64))]
+    outb = torch.empty((qb.shape[0], 4, 128), dtype=qb.dtype, device=dev)
+    kwb = dict(kw, max_seq_len=4096)
+    s1, s2 = torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        hip_backend.mha_fwd(qb, kb, vb, outb, ob, tb, **kwb)
+    with torch.cuda.stream(s2):
+        with pytest.raises(RuntimeError, match="in use"):
+            hip_backend.mha_fwd(q, k, v, out, offs, t, **kw)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s2):  # once the first has finished, the other stream may use the area
+        hip_backend.mha_fwd(q, k, v, out, offs, t, **kw)
+    torch.cuda.synchronize()
+    ref = torch.empty_like(out)
+    hip_backend.mha_fwd(q, k, v, ref, offs, t, **dict(kw, noalloc=False, workspace_bytes=None))
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+
+
 def test_noalloc_entry_point_rejects_what_does_not_fit(pkg, dev):
     """A kv-split whose partial sums exceed the fixed area is refused with its own status, and nothing is written."""
     from generative_recommenders_amd.ops import hip_backend
