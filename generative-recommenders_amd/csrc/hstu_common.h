@@ -420,6 +420,11 @@ __device__ __forceinline__ bool row_block_rows(int nq, int mb, int bm, bool end_
 }
 __device__ __forceinline__ bool row_blocks_end_aligned(const FwdParams& p) { return p.delta == 0 && p.kv_splits <= 1; }
 
+// The pair (sequence in rank order, head) that is number `i` of XCD `xcd`: the pairs are dealt to the XCDs back and
+// forth (0 .. 7, 7 .. 0, ...).  With the sequences ranked by length a plain round-robin gives XCD 0 the longest pair of
+// every eight and XCD 7 the shortest, several per cent more work on the one than on the other.
+__device__ __forceinline__ int pair_of(int i, int xcd) { return i * 8 + ((i & 1) ? 7 - xcd : xcd); }
+
 // x / d for 0 <= x < 2^31 with constants the host derives from d (fast_div_constants in the API source): with
 // l = ceil(log2 d) and m = floor(2^(31+l) / d) + 1, x / d = (x * m) >> (31 + l); magic 0 stands for d = 1.
 __device__ __forceinline__ int fast_div(int x, unsigned magic, unsigned shift) {
@@ -480,7 +485,7 @@ __device__ __forceinline__ bool decode_work(Work& w, int bid) {
             pair_local = fast_div(slot, p.mb_magic, p.mb_shift);
             mb = p.num_mb - 1 - (slot - pair_local * p.num_mb);
         }
-        const int pair = pair_local * 8 + xcd;
+        const int pair = pair_of(pair_local, xcd);
         if (pair >= p.B * p.H) return false;
         const int rseq = fast_div(pair, p.h_magic, p.h_shift);
         w.h = pair - rseq * p.H;
@@ -554,7 +559,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
 
 #define HSTU_PLAN_THREADS 1024
 // Builds the work lists of the persistent kernels: one workgroup per XCD walks the (sequence, head) pairs that
-// XCD owns (pair = 8 * i + xcd, sequences taken in `order` if given) and lists every row block that exists,
+// XCD owns (pair_of(i, xcd), sequences taken in `order` if given) and lists every row block that exists,
 // sorted by weight class (floor(log2(kv tiles)), heaviest class first; within a class in pair order, within a
 // pair heaviest block first).  Heavy-first across the whole list keeps the end of the launch made of small
 // items, items of one class and pair stay neighbours (they share K/V through the L2), and row blocks past the
@@ -594,7 +599,7 @@ static __global__ __launch_bounds__(HSTU_PLAN_THREADS) void hstu_plan_kernel(con
             if (!place && k < CACHE) cls[k] = -1;
             if (pl != cur_pl) {
                 cur_pl = pl;
-                const int pair = pl * 8 + xcd;
+                const int pair = pair_of(pl, xcd);
                 live = pair < p.B * p.H;
                 if (live) {
                     const int rseq = pair / p.H;
