@@ -12,6 +12,7 @@
 #include <mutex>
 #include <tuple>
 
+#include "hstu_philox.h"
 #include "hstu_uqvk_kernel.h"
 #include "hstu_output_kernel.h"
 
@@ -125,7 +126,33 @@ struct NormMulParams {
     int d, group_lanes;                      // row width; lanes per head (group norm)
     int off_u, off_x, off_y;                 // column offsets of the blocks in `joined`, -1 = block absent
     int silu_u, mul_act;
+    hstu::DropoutParams drop;                // thresh 0: no dropout
+    int64_t width;                           // logical width of `joined` (all blocks): the mask's row pitch
 };
+
+// Eight consecutive elements starting at column `col` (a multiple of 8) of row r: dropped or scaled, in fp32.
+template <class V8, class E>
+__device__ __forceinline__ V8 dropout8(const hstu::DropoutParams& d, int64_t r, int64_t width, int64_t col, const float (&x)[8]) {
+    const uint64_t group = (uint64_t)(r * width + col) >> 2;
+    const hstu::PhiloxWords a = hstu::dropout_words(d, group), b = hstu::dropout_words(d, group + 1);
+    V8 out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        out[j] = (E)(a.w[j] >= d.thresh ? x[j] * d.scale : 0.f);
+        out[4 + j] = (E)(b.w[j] >= d.thresh ? x[4 + j] * d.scale : 0.f);
+    }
+    return out;
+}
+
+// keep[r * width + c] = 1 where the element survives: what the backward pass multiplies by (times the scale).
+__global__ __launch_bounds__(256) void hstu_dropout_mask_kernel(hstu::DropoutParams d, int64_t groups, unsigned char* keep) {
+    for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
+        const hstu::PhiloxWords a = hstu::dropout_words(d, (uint64_t)g);
+        uchar4 k;
+        k.x = a.w[0] >= d.thresh, k.y = a.w[1] >= d.thresh, k.z = a.w[2] >= d.thresh, k.w = a.w[3] >= d.thresh;
+        ((uchar4*)keep)[g] = k;
+    }
+}
 
 __device__ __forceinline__ float sigmoid_f(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
@@ -218,7 +245,8 @@ __global__ __launch_bounds__(256) void hstu_norm_mul_kernel(NormMulParams p) {
         for (int i = 0; i < NCH; ++i) {
             const int c = lane + 64 * i;
             if (c < chunks) {
-                V8 y, ucopy = uraw[i];
+                V8 y, ucopy = uraw[i], xcopy = xraw[i];
+                float yf[8], uf32[8];  // y before it is rounded, u in fp32 (used again only when elements are dropped)
                 if (p.silu_u || (!GROUP && p.mul_act != HSTU_MUL_U_NONE)) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
@@ -232,19 +260,44 @@ __global__ __launch_bounds__(256) void hstu_norm_mul_kernel(NormMulParams p) {
                             if (p.mul_act == HSTU_MUL_U_SILU) mul = us;
                         }
                         if (p.silu_u) ucopy[j] = (E)us;
-                        y[j] = (E)(mul * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]));
+                        uf32[j] = uf;
+                        yf[j] = mul * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]);
+                        y[j] = (E)yf[j];
                     }
                 } else {  // no activation anywhere: the exponentials are not worth computing to be thrown away
 #pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        y[j] = (E)((float)uraw[i][j] * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]));
+                    for (int j = 0; j < 8; ++j) {
+                        uf32[j] = (float)uraw[i][j];
+                        yf[j] = uf32[j] * ((v[i][j] - mean[i]) * rstd[i] * w[i][GROUP ? 0 : j] + b[i][GROUP ? 0 : j]);
+                        y[j] = (E)yf[j];
+                    }
+                }
+                if (p.drop.thresh != 0) {
+                    // as the reference: the whole of `joined` goes through dropout, in fp32, before it is rounded
+                    if (p.off_u >= 0) {
+                        float t[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) t[j] = p.silu_u ? uf32[j] * sigmoid_f(uf32[j]) : uf32[j];
+                        ucopy = dropout8<V8, E>(p.drop, r, p.width, (int64_t)p.off_u + c * 8, t);
+                    }
+                    if (p.off_x >= 0) xcopy = dropout8<V8, E>(p.drop, r, p.width, (int64_t)p.off_x + c * 8, v[i]);
+                    y = dropout8<V8, E>(p.drop, r, p.width, (int64_t)p.off_y + c * 8, yf);
                 }
                 if (p.off_u >= 0) *(V8*)(orow + ((int64_t)p.off_u + c * 8) * 2) = ucopy;
-                if (p.off_x >= 0) *(V8*)(orow + ((int64_t)p.off_x + c * 8) * 2) = xraw[i];
+                if (p.off_x >= 0) *(V8*)(orow + ((int64_t)p.off_x + c * 8) * 2) = xcopy;
                 *(V8*)(orow + ((int64_t)p.off_y + c * 8) * 2) = y;
             }
         }
     }
+}
+
+// False: the ratio is not in [0, 1).
+bool dropout_params(float ratio, uint64_t seed, uint64_t offset, hstu::DropoutParams& d) {
+    if (!(ratio >= 0.f && ratio < 1.f)) return false;
+    d.seed = seed, d.offset = offset;
+    d.thresh = (uint32_t)((double)ratio * 4294967296.0);
+    d.scale = 1.0f / (1.0f - ratio);
+    return true;
 }
 
 int output_blocks(const HstuOutputArgs* a) {
@@ -270,7 +323,7 @@ bool output_fused_u_made(const HstuOutputArgs* a) { return !a->group_norm && a->
 // path = 0: the concatenating path where it applies and the rows fill the chip (a workgroup takes 256 rows x 256 columns;
 // measured against the library path it wins from 32768 rows on: 70 against 77 us there, 37 against 32 us at 2048).
 bool output_takes_fused(const HstuOutputArgs* a) {
-    return a->path == 2 || (a->path == 0 && a->rows >= 32768 && output_fused_shape(a));
+    return a->path == 2 || (a->path == 0 && a->rows >= 32768 && a->dropout_ratio == 0.f && output_fused_shape(a));
 }
 
 size_t output_fused_workspace(const HstuOutputArgs* a) {
@@ -352,6 +405,8 @@ int launch_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_rs, hi
     p.off_x = cx ? (cu ? d : 0) : -1;
     p.off_y = (blocks - 1) * d;
     p.silu_u = a->silu_u ? 1 : 0, p.mul_act = a->mul_u_activation;
+    p.width = (int64_t)blocks * d;
+    if (!dropout_params(a->dropout_ratio, a->dropout_seed, a->dropout_offset, p.drop)) return -5;
     long long wgs = (a->rows + 3) / 4;
     if (wgs > 256 * 16) wgs = 256 * 16;
     const int nch = (d / 8 + 63) / 64;
@@ -693,6 +748,25 @@ int hstu_output_norm_mul(const HstuOutputArgs* a, void* joined, int64_t joined_r
     return launch_norm_mul(a, joined, joined_row_stride, (hipStream_t)stream);
 }
 
+int hstu_output_dropout_mask(float ratio, uint64_t seed, uint64_t offset, int64_t rows, int64_t width, void* keep, void* stream) {
+    g_last_error[0] = 0;
+    hstu::DropoutParams d;
+    if (rows < 0 || width < 0 || (width & 7) != 0 || !dropout_params(ratio, seed, offset, d)) return -5;
+    if (rows == 0 || width == 0) return 0;
+    if (!keep) return -1;
+    if (((uintptr_t)keep & 3) != 0) return -4;
+    const int64_t groups = rows * width / 4;
+    long long wgs = (groups + 255) / 256;
+    if (wgs > 256 * 16) wgs = 256 * 16;
+    hipLaunchKernelGGL(hstu_dropout_mask_kernel, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, d, groups, (unsigned char*)keep);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        snprintf(g_last_error, sizeof(g_last_error), "dropout mask kernel launch: %s", hipGetErrorString(e));
+        return -7;
+    }
+    return 0;
+}
+
 int hstu_output_forward(const HstuOutputArgs* a, void* stream_) {
     g_last_error[0] = 0;
     if (!a) return -1;
@@ -706,6 +780,11 @@ int hstu_output_forward(const HstuOutputArgs* a, void* stream_) {
     if (a->path == 2 && !output_fused_shape(a)) {
         snprintf(g_last_error, sizeof(g_last_error), "the concatenating output kernel takes d_out a multiple of 256 and heads * linear_dim a multiple "
                  "of 64 up to 4096, row strides below 2^22 (and, with group norm, no SiLU on a copied u)");
+        return -6;
+    }
+    if (a->dropout_ratio != 0.f && a->path == 2) {
+        snprintf(g_last_error, sizeof(g_last_error), "the concatenating output kernel reads u and attn where they are and cannot drop their "
+                 "elements: dropout runs on the library path (path 0 or 1)");
         return -6;
     }
     if (output_takes_fused(a)) {

@@ -357,10 +357,6 @@ def mha_bwd_workspace_bytes(total_rows: int, batch: int, heads: int, max_seq_len
     return int(lib().hstu_hip_mha_bwd_workspace_bytes(ctypes.byref(a)))
 
 
-# Largest dS scratch mha_bwd takes by itself (the caching allocator keeps it between calls).
-BWD_SCRATCH_LIMIT_BYTES = 40 << 30
-
-
 def mha_bwd(
     dout: torch.Tensor,
     q: torch.Tensor,
@@ -377,16 +373,18 @@ def mha_bwd(
     contextual_seq_len: int,
     min_full_attn_seq_len: int,
     sort_by_length: bool = True,
-    store_ds: Optional[bool] = None,
+    store_ds: bool = False,
     workspace: Optional[torch.Tensor] = None,
 ) -> None:
     """Fill ``dq``, ``dk``, ``dv`` on the current stream of ``q.device`` (full attention only).  ``sort_by_length``
-    starts the long sequences first; it never changes the result.  ``store_ds``: let the kernel that forms dk and dv
-    write dS to scratch memory (2 bytes per query row, head and key position up to ``max_seq_len``) so that dq is one
-    streamed product instead of a second pass over the scores; ``None`` = when that scratch is at most
-    ``BWD_SCRATCH_LIMIT_BYTES`` and half of the device's free memory.  ``workspace``: the caller's own scratch (uint8,
-    256-byte aligned; ``mha_bwd_workspace_bytes`` says how much the stored form takes) instead of a fresh allocation;
-    it decides the form by its size."""
+    starts the long sequences first; it never changes the result.
+
+    Two forms, chosen by the caller and by nothing else (not by how much device memory happens to be free).  The
+    default recomputes the scores for dq and needs no scratch beyond ``4 * batch`` bytes for the sort.  The stored
+    form lets the kernel that forms dk and dv write dS to scratch memory (2 bytes per query row, head and key position
+    up to ``max_seq_len``; ``mha_bwd_workspace_bytes`` says how much), so that dq is one streamed product instead of a
+    second pass over the scores: it runs when the caller passes a ``workspace`` of that size (uint8, 256-byte aligned;
+    a smaller one selects the recomputed form) or asks for a fresh allocation with ``store_ds=True``."""
     a = HstuFwdArgs()
     a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), None
     a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
@@ -413,14 +411,8 @@ def mha_bwd(
         a.sort_by_length = 1 if sort_by_length else 0
     else:
         need = 4 * a.batch if sort_by_length and a.batch >= 2 else 0
-        if store_ds is not False and a.total_q > 0 and a.batch > 0:
-            stored = lib().hstu_hip_mha_bwd_workspace_bytes(ctypes.byref(a))
-            if store_ds is None:
-                store_ds = stored <= BWD_SCRATCH_LIMIT_BYTES
-                if store_ds and not torch.cuda.is_current_stream_capturing():
-                    store_ds = 2 * stored <= torch.cuda.mem_get_info(q.device)[0]
-            if store_ds:
-                need = stored
+        if store_ds and a.total_q > 0 and a.batch > 0:
+            need = lib().hstu_hip_mha_bwd_workspace_bytes(ctypes.byref(a))
         if need:
             workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
             a.workspace, a.workspace_bytes, a.sort_by_length = workspace.data_ptr(), need, 1 if sort_by_length else 0

@@ -57,7 +57,7 @@ class _HstuMhaFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
-                min_full_attn_seq_len, sort_by_length, tile_config, kv_splits, attn_scale):
+                min_full_attn_seq_len, sort_by_length, tile_config, kv_splits, attn_scale, bwd_workspace):
         q, k, v = _kernel_layout(q.detach()), _kernel_layout(k.detach()), _kernel_layout(v.detach())
         out = torch.empty((v.shape[0], v.shape[1], v.shape[2]), dtype=v.dtype, device=v.device)
         if out.numel() > 0:
@@ -69,6 +69,7 @@ class _HstuMhaFunction(torch.autograd.Function):
         ctx.save_for_backward(q, k, v, seq_offsets, *([] if num_targets is None else [num_targets]))
         ctx.has_targets = num_targets is not None
         ctx.attn_scale = attn_scale  # a constant of the call (no gradient flows into it)
+        ctx.bwd_workspace = bwd_workspace  # the caller's dS scratch, or None: the backward recomputes the scores
         ctx.params = (max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len)
         return out
 
@@ -95,11 +96,11 @@ class _HstuMhaFunction(torch.autograd.Function):
             dout = _kernel_layout(dout.detach().to(q.dtype))
             hip_backend.mha_bwd(
                 dout, q, k, v, dq, dk, dv, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len,
-                min_full_attn_seq_len,
+                min_full_attn_seq_len, workspace=ctx.bwd_workspace,
             )
         if wide:
             dq, dk, dv = dq.float(), dk.float(), dv.float()
-        return (dq, dk, dv) + (None,) * 11
+        return (dq, dk, dv) + (None,) * 12
 
 
 def _require_device(t: torch.Tensor, name: str) -> None:
@@ -146,6 +147,7 @@ def hstu_mha(
     v_scale: float = 1.0,
     tile_config: int = 0,
     kv_splits: int = 0,
+    bwd_workspace: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Jagged HSTU attention forward; returns ``[L, H, Dv]``.
 
@@ -157,6 +159,10 @@ def hstu_mha(
     rows of a sequence that breaks it may come back UNINITIALISED (the output is ``torch.empty``).  Set
     ``HSTU_HIP_CHECK_CONTRACT=1`` in the environment to have every call validated on the device first and raise
     ``ValueError`` instead.
+
+    The backward recomputes the scores and allocates nothing that grows with ``max_seq_len``.  ``bwd_workspace`` (uint8,
+    ``hip_backend.mha_bwd_workspace_bytes`` bytes, kept by the caller across steps) selects the faster form that stores
+    dS there; the choice never depends on how much device memory is free.
     """
     torch._assert(max_seq_len > 0, "max_seq_len must be larger than 0")
     torch._assert(q.dim() == 3, "q must be 3-D")
@@ -189,7 +195,7 @@ def hstu_mha(
             _check_forward_only(q, k, v)
         return _HstuMhaFunction.apply(
             q, k, v, seq_offsets, num_targets, max_seq_len, alpha, max_attn_len, contextual_seq_len, min_full_attn_seq_len,
-            sort_by_length, tile_config, kv_splits, attn_scale,
+            sort_by_length, tile_config, kv_splits, attn_scale, bwd_workspace,
         )
 
     q = _kernel_layout(q.detach())

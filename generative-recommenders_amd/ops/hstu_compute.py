@@ -77,12 +77,15 @@ class HstuOutputArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
         ("path", ctypes.c_int32),
+        ("dropout_ratio", ctypes.c_float),
+        ("dropout_seed", ctypes.c_uint64),
+        ("dropout_offset", ctypes.c_uint64),
     ]
 
 
 EXPORTS = (
     "hstu_uqvk_workspace_bytes", "hstu_uqvk_forward", "hstu_uqvk_layer_norm", "hstu_output_workspace_bytes", "hstu_output_forward",
-    "hstu_output_norm_mul", "hstu_linear_last_error",
+    "hstu_output_norm_mul", "hstu_output_dropout_mask", "hstu_linear_last_error",
 )
 MUL_U_ACTIVATIONS = {"none": 0, "sigmoid": 1, "silu": 2}
 
@@ -111,6 +114,9 @@ def lib() -> ctypes.CDLL:
         L.hstu_output_forward.argtypes = [ctypes.POINTER(HstuOutputArgs), ctypes.c_void_p]
         L.hstu_output_norm_mul.restype = ctypes.c_int
         L.hstu_output_norm_mul.argtypes = [ctypes.POINTER(HstuOutputArgs), ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+        L.hstu_output_dropout_mask.restype = ctypes.c_int
+        L.hstu_output_dropout_mask.argtypes = [ctypes.c_float, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int64, ctypes.c_int64,
+                                               ctypes.c_void_p, ctypes.c_void_p]
         L.hstu_linear_last_error.restype = ctypes.c_char_p
         _lib = L
     return _lib
@@ -166,7 +172,9 @@ def _uqvk_math(x, norm_weight, norm_bias, eps, u_cols, weight, bias):
     return torch.cat([F.silu(uvqk[:, :u_cols]), uvqk[:, u_cols:]], dim=1)
 
 
-def _norm_mul_math(attn, u, weight, bias, eps, silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim):
+def _norm_mul_math(attn, u, weight, bias, eps, silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim, keep_scaled=None):
+    """The output step's first half with the framework's operators (for the backward's recomputation).  ``keep_scaled``:
+    the dropout mask times ``1 / (1 - p)`` in fp32, applied to the whole concatenation before it is rounded."""
     a32, u32, w32, b32 = attn.float(), u.float(), weight.float(), bias.float()
     if group_norm:
         if silu_u:
@@ -182,7 +190,10 @@ def _norm_mul_math(attn, u, weight, bias, eps, silu_u, concat_u, concat_x, act, 
         gate = torch.sigmoid(u32) if act == "sigmoid" else F.silu(u32) if act == "silu" else u32
         y = gate * F.layer_norm(a32, (a32.shape[-1],), w32, b32, eps)
         parts = ([F.silu(u32) if silu_u else u32] if concat_u else []) + ([a32] if concat_x else []) + [y]
-    return (torch.cat(parts, dim=1) if len(parts) > 1 else parts[0]).to(attn.dtype)
+    joined = torch.cat(parts, dim=1) if len(parts) > 1 else parts[0]
+    if keep_scaled is not None:
+        joined = joined * keep_scaled
+    return joined.to(attn.dtype)
 
 
 def _grads_by_recomputation(fn, tensors, d_out):
@@ -337,65 +348,119 @@ def _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_di
     return a, (attn, u, nw, nb), blocks
 
 
-def _no_dropout(dropout_ratio: float, training: bool) -> None:
-    if training and dropout_ratio > 0.0:
-        raise NotImplementedError("the HIP backend implements the dropout-free forward only (training=False or dropout_ratio=0)")
+def _dropout_state(dropout_ratio: float, training: bool, elements: int, device: torch.device, seed) -> Optional[Tuple[float, int, int]]:
+    """``None`` when nothing is dropped, else ``(ratio, seed, offset)`` of the Philox stream the kernel draws the mask from:
+    the caller's ``seed = (seed, offset)``, or the device's default generator, advanced past the words this call uses (one
+    word per element) as the framework's own dropout would advance it."""
+    if not training or dropout_ratio <= 0.0:
+        return None
+    torch._assert(dropout_ratio < 1.0, "dropout_ratio must be below 1")
+    if seed is not None:
+        return float(dropout_ratio), int(seed[0]), int(seed[1])
+    gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+    offset = gen.get_offset()
+    gen.set_offset(offset + ((elements + 3) // 4 + 3) // 4 * 4)
+    return float(dropout_ratio), gen.initial_seed(), offset
+
+
+def dropout_keep_mask(state: Tuple[float, int, int], rows: int, width: int, device: torch.device) -> torch.Tensor:
+    """``[rows, width]`` uint8, 1 where the dropout of a call with this ``(ratio, seed, offset)`` kept the element: the mask
+    is a pure function of these and of the element's position, regenerated on the device whenever it is needed."""
+    keep = torch.empty((rows, width), dtype=torch.uint8, device=device)
+    if keep.numel() > 0:
+        with torch.cuda.device(device):
+            stream = torch.cuda.current_stream(device).cuda_stream
+            rc = lib().hstu_output_dropout_mask(state[0], state[1], state[2], rows, width, keep.data_ptr(), ctypes.c_void_p(stream))
+        _raise_for_status(rc)
+    return keep
+
+
+def _keep_scaled(state, rows: int, width: int, device: torch.device) -> Optional[torch.Tensor]:
+    if state is None:
+        return None
+    # the kernel's factor: 1 / (1 - p) in fp32
+    scale = (torch.ones((), dtype=torch.float32) / (torch.ones((), dtype=torch.float32) - torch.tensor(state[0], dtype=torch.float32))).item()
+    return dropout_keep_mask(state, rows, width, device).float() * scale
+
+
+def _set_dropout(a: HstuOutputArgs, state) -> None:
+    if state is not None:
+        a.dropout_ratio, a.dropout_seed, a.dropout_offset = state
 
 
 class _NormMulFunction(torch.autograd.Function):
+    """Saves the inputs and the dropout stream's ``(ratio, seed, offset)``; the backward recomputes ``joined`` with the
+    mask regenerated on the device."""
+
     @staticmethod
-    def forward(ctx, x, u, weight, bias, eps, *flags):
+    def forward(ctx, x, u, weight, bias, eps, state, *flags):
         ctx.save_for_backward(x, u, weight, bias)
         ctx.cfg = (eps,) + flags
-        silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim = flags
+        ctx.state = state
         with torch.no_grad():
-            return norm_mul_dropout(x, u, weight, bias, eps, 0.0, False, silu_u, concat_u, concat_x, act, group_norm, heads, linear_dim)
+            return _norm_mul_forward(x, u, weight, bias, eps, state, *flags)
 
     @staticmethod
     def backward(ctx, d_out):
         cfg = ctx.cfg
-        fn = lambda x, u, w, b: _norm_mul_math(x, u, w, b, *cfg)  # noqa: E731
-        return _grads_by_recomputation(fn, ctx.saved_tensors, d_out.contiguous()) + (None,) * 8
+        x = ctx.saved_tensors[0]
+        mask = _keep_scaled(ctx.state, d_out.shape[0], d_out.shape[1], x.device)
+        fn = lambda x, u, w, b: _norm_mul_math(x, u, w, b, *cfg, keep_scaled=mask)  # noqa: E731
+        return _grads_by_recomputation(fn, ctx.saved_tensors, d_out.contiguous()) + (None,) * 9
 
 
 class _OutputFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, attn, u, x, norm_weight, norm_bias, output_weight, norm_eps, num_heads, linear_dim, concat_u, concat_x, act,
-                group_norm, path):
+                group_norm, path, state):
         ctx.save_for_backward(attn, u, x, norm_weight, norm_bias, output_weight)
         ctx.cfg = (norm_eps, False, concat_u, concat_x, act, group_norm, num_heads, linear_dim)
+        ctx.state = state
         with torch.no_grad():
-            return hstu_compute_output(attn, u, x, norm_weight, norm_bias, norm_eps, output_weight, num_heads, linear_dim, 0.0, False,
-                                       concat_u, concat_x, act, group_norm, False, path=path)
+            return _output_forward(attn, u, x, norm_weight, norm_bias, norm_eps, output_weight, num_heads, linear_dim, concat_u,
+                                   concat_x, act, group_norm, path, state)
 
     @staticmethod
     def backward(ctx, d_out):
         cfg = ctx.cfg
-        fn = lambda attn, u, x, nw, nb, w: torch.addmm(x, _norm_mul_math(attn, u, nw, nb, *cfg), w)  # noqa: E731
-        return _grads_by_recomputation(fn, ctx.saved_tensors, d_out.contiguous()) + (None,) * 8
+        attn, w = ctx.saved_tensors[0], ctx.saved_tensors[5]
+        mask = _keep_scaled(ctx.state, attn.shape[0], w.shape[0], attn.device)
+        fn = lambda attn, u, x, nw, nb, w: torch.addmm(x, _norm_mul_math(attn, u, nw, nb, *cfg, keep_scaled=mask), w)  # noqa: E731
+        return _grads_by_recomputation(fn, ctx.saved_tensors, d_out.contiguous()) + (None,) * 9
 
 
-def norm_mul_dropout(
-    x: torch.Tensor, u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, dropout_ratio: float, training: bool,
-    silu_u: bool = False, concat_u: bool = False, concat_x: bool = False, mul_u_activation_type: str = "none",
-    group_norm: bool = False, num_heads: int = 1, linear_dim: int = -1,
-) -> torch.Tensor:
-    """``act(u) * norm(x)`` joined with the copied blocks (``ops/pytorch/pt_hstu_linear.py:24-85`` of the reference),
-    without dropout."""
-    _no_dropout(dropout_ratio, training)
-    _check(x, u, weight, bias)
-    if not group_norm:
-        num_heads, linear_dim = 1, x.shape[1]
-    if _needs_grad(x, u, weight, bias):
-        return _NormMulFunction.apply(x, u, weight, bias, eps, silu_u, concat_u, concat_x, mul_u_activation_type, group_norm,
-                                      num_heads, linear_dim)
-    a, keep, blocks = _output_args(x, u, weight, bias, eps, num_heads, linear_dim, concat_u, concat_x, mul_u_activation_type, group_norm, silu_u)
+def _norm_mul_forward(x, u, weight, bias, eps, state, silu_u, concat_u, concat_x, act, group_norm, num_heads, linear_dim) -> torch.Tensor:
+    a, keep, blocks = _output_args(x, u, weight, bias, eps, num_heads, linear_dim, concat_u, concat_x, act, group_norm, silu_u)
+    _set_dropout(a, state)
     joined = torch.empty((x.shape[0], blocks * x.shape[1]), dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream(x.device).cuda_stream
         rc = lib().hstu_output_norm_mul(ctypes.byref(a), joined.data_ptr(), joined.shape[1], ctypes.c_void_p(stream))
     _raise_for_status(rc)
     return joined
+
+
+def _blocks(concat_u: bool, concat_x: bool, group_norm: bool) -> int:
+    return (3 if (concat_u and concat_x) else 1) if group_norm else 1 + int(concat_u) + int(concat_x)
+
+
+def norm_mul_dropout(
+    x: torch.Tensor, u: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, dropout_ratio: float, training: bool,
+    silu_u: bool = False, concat_u: bool = False, concat_x: bool = False, mul_u_activation_type: str = "none",
+    group_norm: bool = False, num_heads: int = 1, linear_dim: int = -1, seed: Optional[Tuple[int, int]] = None,
+) -> torch.Tensor:
+    """``dropout(act(u) * norm(x) joined with the copied blocks)`` (``ops/pytorch/pt_hstu_linear.py:24-85`` of the
+    reference).  Dropout runs when ``training`` and ``dropout_ratio > 0``, over the whole concatenation, in fp32 before the
+    result is rounded; its mask comes from a Philox stream -- ``seed = (seed, offset)``, or the device's default
+    generator -- and is regenerated, not stored, for the backward."""
+    _check(x, u, weight, bias)
+    if not group_norm:
+        num_heads, linear_dim = 1, x.shape[1]
+    state = _dropout_state(dropout_ratio, training, x.shape[0] * x.shape[1] * _blocks(concat_u, concat_x, group_norm), x.device, seed)
+    flags = (silu_u, concat_u, concat_x, mul_u_activation_type, group_norm, num_heads, linear_dim)
+    if _needs_grad(x, u, weight, bias):
+        return _NormMulFunction.apply(x, u, weight, bias, eps, state, *flags)
+    return _norm_mul_forward(x, u, weight, bias, eps, state, *flags)
 
 
 def hstu_compute_output(
@@ -417,21 +482,30 @@ def hstu_compute_output(
     recompute_y_in_backward: bool,
     kernel: HammerKernel = HammerKernel.HIP,
     path: int = 0,
+    seed: Optional[Tuple[int, int]] = None,
 ) -> torch.Tensor:
-    """Returns ``x + joined @ output_weight`` of shape ``[L, d_model]``.  The backward always recomputes ``joined``
+    """Returns ``x + dropout(joined) @ output_weight`` of shape ``[L, d_model]``.  The backward always recomputes ``joined``
     (what ``recompute_y_in_backward=True`` asks for), so the flag changes nothing.  ``path``: 1 = the norm-mul kernel
     writes ``joined`` and hipBLASLt multiplies it; 2 = the norm-mul kernel writes ``y`` alone and a hand-written GEMM
     reads ``u`` and ``attn`` where they are (``NotImplementedError`` if the shape does not fit: d_model a multiple of 256,
-    heads * linear_dim a multiple of 64); 0 = whichever is faster for the shape (2 where it fits and rows >= 32768)."""
-    _no_dropout(dropout_ratio, training)
+    heads * linear_dim a multiple of 64 -- or with dropout, whose mask covers the copied blocks too); 0 = whichever is
+    faster for the shape (2 where it fits, rows >= 32768 and nothing is dropped).  Dropout as in ``norm_mul_dropout``."""
     torch._assert(x.dim() == 2 and x.shape[0] == attn.shape[0], "x must be 2-D with attn's row count")
     _check(x, attn, u, norm_weight, norm_bias, output_weight)
+    torch._assert(mul_u_activation_type in MUL_U_ACTIVATIONS, "mul_u_activation_type must be none, sigmoid or silu")
+    state = _dropout_state(dropout_ratio, training, attn.shape[0] * attn.shape[1] * _blocks(concat_u, concat_x, group_norm), attn.device, seed)
     if _needs_grad(x, attn, u, norm_weight, norm_bias, output_weight):
-        torch._assert(mul_u_activation_type in MUL_U_ACTIVATIONS, "mul_u_activation_type must be none, sigmoid or silu")
         return _OutputFunction.apply(attn, u, x, norm_weight, norm_bias, output_weight, norm_eps, num_heads, linear_dim, concat_u,
-                                     concat_x, mul_u_activation_type, group_norm, path)
+                                     concat_x, mul_u_activation_type, group_norm, path, state)
+    return _output_forward(attn, u, x, norm_weight, norm_bias, norm_eps, output_weight, num_heads, linear_dim, concat_u, concat_x,
+                           mul_u_activation_type, group_norm, path, state)
+
+
+def _output_forward(attn, u, x, norm_weight, norm_bias, norm_eps, output_weight, num_heads, linear_dim, concat_u, concat_x,
+                    mul_u_activation_type, group_norm, path, state) -> torch.Tensor:
     a, keep, blocks = _output_args(attn, u, norm_weight, norm_bias, norm_eps, num_heads, linear_dim, concat_u, concat_x,
                                    mul_u_activation_type, group_norm, False)
+    _set_dropout(a, state)
     torch._assert(output_weight.shape == (blocks * attn.shape[1], x.shape[1]), "output_weight must be [blocks * heads * linear_dim, d_model]")
     xr, w = _rows_ok(x), _dense16(output_weight)
     out = torch.empty((x.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)

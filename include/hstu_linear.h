@@ -68,8 +68,8 @@ int hstu_uqvk_layer_norm(const void* x, int64_t x_row_stride, const void* weight
                          int64_t out_row_stride, int64_t rows, int32_t d_model, int32_t dtype, void* stream);
 
 /*
- * Consumer: replaces `hstu_compute_output` (generative_recommenders/ops/hstu_compute.py:107-214) in its forward,
- * dropout-free form, i.e. `pytorch_hstu_compute_output` (ops/pytorch/pt_hstu_linear.py:88-124):
+ * Consumer: replaces `hstu_compute_output` (generative_recommenders/ops/hstu_compute.py:107-214) in its forward
+ * form, i.e. `pytorch_hstu_compute_output` (ops/pytorch/pt_hstu_linear.py:88-124); dropout: see `dropout_ratio`:
  *     y   = norm_mul(attn, u)                      (pt_hstu_linear.py:24-85, statistics and product in fp32)
  *              layer norm : y = act(u) * layer_norm(attn) over the whole row, act in {none, sigmoid, silu};
  *                           joined = [u] | [attn] | y, a block present when concat_u / concat_x is set
@@ -111,6 +111,14 @@ typedef struct HstuOutputArgs {
                                   + hand-written GEMM over the blocks where they are): needs d_out a multiple of 256 and heads *
                                   linear_dim a multiple of 64 (and, with group norm, no SiLU on a copied u), else status
                                   -6; 0 = the concatenating path where it applies and rows >= 32768, else the library */
+    /* Dropout of `joined` (`F.dropout(y, p, training)` at the end of pytorch_norm_mul_dropout, pt_hstu_linear.py:80-84): the
+     * whole concatenation goes through it, in fp32, before it is rounded; survivors are multiplied by 1 / (1 - ratio).
+     * Element (r, c) of the [rows, blocks * heads * linear_dim] matrix is kept when word c % 4 of
+     * Philox4x32-10(counter = {(r * width + c) / 4, dropout_offset}, key = dropout_seed) is >= floor(ratio * 2^32): a pure
+     * function of (seed, offset, r, c), so hstu_output_dropout_mask returns the mask of any earlier call.  0 = no
+     * dropout (inference, `training=False`); with a ratio > 0 path 2 is refused (-6) and path 0 takes the library path. */
+    float dropout_ratio;       /* [0, 1) */
+    uint64_t dropout_seed, dropout_offset;
 } HstuOutputArgs;
 
 size_t hstu_output_workspace_bytes(const HstuOutputArgs* args);
@@ -118,10 +126,16 @@ size_t hstu_output_workspace_bytes(const HstuOutputArgs* args);
 /* norm_mul + concatenation + GEMM + residual, as described above. */
 int hstu_output_forward(const HstuOutputArgs* args, void* stream);
 
-/* Only the first step (`pytorch_norm_mul_dropout` without dropout, pt_hstu_linear.py:24-85): writes `joined`
+/* Only the first step (`pytorch_norm_mul_dropout`, pt_hstu_linear.py:24-85): writes `joined`
  * [rows, blocks * heads * linear_dim] with row stride `joined_row_stride` elements.  Reads attn, u, norm_weight,
- * norm_bias, norm_eps, rows, heads, linear_dim, the five flags and dtype of `args`; the other fields are ignored. */
+ * norm_bias, norm_eps, rows, heads, linear_dim, the five flags, dtype and the dropout fields of `args`; the other fields are
+ * ignored. */
 int hstu_output_norm_mul(const HstuOutputArgs* args, void* joined, int64_t joined_row_stride, void* stream);
+
+/* keep[r * width + c] (one byte per element, 1 = kept) for the mask a call with the same ratio, seed and offset applied to a
+ * `joined` of `width` columns (a multiple of 8): what the backward of the dropout multiplies by, times 1 / (1 - ratio).
+ * `keep`: rows * width bytes of device memory, 4-byte aligned. */
+int hstu_output_dropout_mask(float ratio, uint64_t seed, uint64_t offset, int64_t rows, int64_t width, void* keep, void* stream);
 
 const char* hstu_linear_last_error(void);
 

@@ -149,19 +149,20 @@ def _poisoned_workspace(dev, q, offsets, N):
 
 
 def _check(pkg, dev, N, alpha, q, k, v, dout, offsets, what, **kw):
-    """Both forms of the backward against the closed form: dS stored (through autograd, and through the entry point on
-    NaN-filled scratch) and scores recomputed; dk and dv do not depend on the form."""
+    """Both forms of the backward against the closed form: scores recomputed (through autograd, whose default it is, and
+    through the entry point) and dS stored (through the entry point on NaN-filled scratch); dk and dv do not depend on
+    the form."""
     out, dq, dk, dv = _run_bwd(pkg, dev, N, alpha, q, k, v, dout, offsets, **kw)
     rq, rk, rv = G.closed_form_grads(N, alpha, q, k, v, offsets, dout, **kw)
     _close(dq, rq, what + " dq")
     _close(dk, rk, what + " dk")
     _close(dv, rv, what + " dv")
     if q.shape[0] > 0:
+        cq, ck, cv = _direct(dev, N, alpha, q, k, v, dout, offsets, kw)
+        assert torch.equal(cq, dq) and torch.equal(ck, dk) and torch.equal(cv, dv), what + ": autograd runs the recomputed form"
         sq, sk, sv = _direct(dev, N, alpha, q, k, v, dout, offsets, kw, workspace=_poisoned_workspace(dev, q, offsets, N))
-        assert torch.equal(sq, dq) and torch.equal(sk, dk) and torch.equal(sv, dv), what + ": stored form on poisoned scratch"
-        cq, ck, cv = _direct(dev, N, alpha, q, k, v, dout, offsets, kw, store_ds=False)
-        _close(cq, rq, what + " dq recomputed")
-        assert torch.equal(ck, dk) and torch.equal(cv, dv), what + ": dk, dv of the two forms"
+        _close(sq, rq, what + " dq from stored dS on poisoned scratch")
+        assert torch.equal(sk, dk) and torch.equal(sv, dv), what + ": dk, dv of the two forms"
     return dq, dk, dv
 
 
@@ -254,6 +255,39 @@ def test_backward_through_the_backend_entry_point(pkg, dev, ci, store_ds):
     got = _direct(dev, N, alpha, q, k, v, dout, offsets, kw, **how)
     for name, x, r in zip(("dq", "dk", "dv"), got, ref):
         _close(x, r, name)
+
+
+@pytest.mark.gpu
+def test_autograd_backward_form_is_the_callers_choice(pkg, dev):
+    """Without a workspace the backward recomputes the scores and allocates nothing that grows with max_seq_len; with the
+    caller's workspace it stores dS there (the NaN filling is overwritten).  Same gradients to the kernels' rounding."""
+    from generative_recommenders_amd.ops import hip_backend
+
+    print("[case] bwd autograd workspace", flush=True)
+    lengths = [700, 300, 513]
+    q, k, v, dout, offsets = _inputs(77, lengths, 2, 64, 64, torch.bfloat16)
+    N = 1024
+    need = hip_backend.mha_bwd_workspace_bytes(q.shape[0], len(lengths), 2, N)
+    grads = {}
+    for form in ("recomputed", "stored"):
+        ws = None
+        if form == "stored":
+            ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=dev)
+        qd, kd, vd = (t.to(dev).detach().requires_grad_() for t in (q, k, v))
+        out = pkg.hstu_mha(N, 0.125, qd, kd, vd, offsets.to(dev), bwd_workspace=ws)
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats(dev)
+        before = torch.cuda.memory_allocated(dev)
+        out.backward(dout.to(dev))
+        torch.cuda.synchronize()
+        grown = torch.cuda.max_memory_allocated(dev) - before
+        # three gradients, a bf16 copy of dout and the sort's 4 bytes per sequence; never the dS scratch
+        assert grown < need // 4, (form, grown, need)
+        if ws is not None:
+            assert int((ws != 0xFF).sum()) > need // 8  # dS was written into the caller's memory
+        grads[form] = (qd.grad.float().cpu(), kd.grad.float().cpu(), vd.grad.float().cpu())
+    for name, a, b in zip(("dq", "dk", "dv"), grads["recomputed"], grads["stored"]):
+        _close(a, b, name)
 
 
 @pytest.mark.gpu

@@ -88,6 +88,41 @@ def test_oracle_output_with_a_selecting_weight():
 # ---------------------------------------------------------------- GPU
 
 
+def test_oracle_philox_known_answers():
+    """The known-answer vectors of the generator's authors (Random123, kat_vectors, philox4x32 with 10 rounds)."""
+    import numpy as np
+
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+        ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+        ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0], [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+    ]
+    for ctr, key, want in kat:
+        assert O.philox4x32_10(np.array([ctr], dtype=np.uint32), np.array(key, dtype=np.uint32))[0].tolist() == want
+    # rows of a batch are independent of each other
+    both = O.philox4x32_10(np.array([kat[0][0], kat[2][0]], dtype=np.uint32), np.array([kat[0][1], kat[2][1]], dtype=np.uint32))
+    assert both[0].tolist() == kat[0][2] and both[1].tolist() == kat[2][2]
+
+
+@pytest.mark.parametrize("p", [0.1, 0.5])
+def test_oracle_dropout_rate_scale_and_position(p):
+    """Keep rate within three standard deviations; survivors are the fp32 values times 1 / (1 - p), the rest zero; the mask
+    depends on seed, offset and position only (a wider matrix re-deals it, another offset gives another mask)."""
+    rows, width = 512, 256
+    keep = O.dropout_keep(p, 1234, 8, rows, width)
+    n = rows * width
+    assert abs(int(keep.sum()) - n * (1 - p)) <= 3 * (n * p * (1 - p)) ** 0.5
+    y = torch.rand((rows, width), generator=torch.Generator().manual_seed(1)) + 0.5
+    d = O.dropout(y, p, 1234, 8)
+    k = torch.from_numpy(keep)
+    assert torch.equal(d[~k], torch.zeros_like(d[~k]))
+    scale = torch.tensor(1.0, dtype=torch.float32) / (torch.tensor(1.0, dtype=torch.float32) - torch.tensor(p, dtype=torch.float32))
+    assert torch.equal(d[k], y[k] * scale)
+    assert (O.dropout_keep(p, 1234, 12, rows, width) != keep).any() and (O.dropout_keep(p, 1235, 8, rows, width) != keep).any()
+    assert (O.dropout_keep(p, 1234, 8, rows // 2, width * 2).reshape(rows, width) == keep).all()  # element index = r * width + c
+
+
+
 @pytest.fixture(scope="module")
 def pkg():
     import __graft_entry__
@@ -341,8 +376,8 @@ def test_output_takes_strided_views_and_rejects_what_it_cannot_do(pkg, dev):
                                   ld, 0.0, False, True, True, "none", False, False)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
-    with pytest.raises(NotImplementedError):
-        pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, ld, 0.3, True, True, True, "none", False, False)
+    with pytest.raises(AssertionError):  # a ratio of 1 would drop everything and scale by infinity
+        pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w, H, ld, 1.0, True, True, True, "none", False, False)
     with pytest.raises(AssertionError):
         pkg.hstu_compute_output(attn, u, x, nw, nb, 1e-6, w[:-8], H, ld, 0.0, False, True, True, "none", False, False)
     with pytest.raises(AssertionError):
@@ -470,3 +505,88 @@ def test_one_layer_training_step(pkg, dev):
         got, want = h.grad.float().cpu(), r.grad
         rel = float((got - want).norm() / want.norm())
         assert rel <= 3e-2, f"d/d{name}: relative {rel:.3e}"
+
+
+# ---------------------------------------------------------------- dropout
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("p", [0.1, 0.5])
+@pytest.mark.parametrize("group_norm", [False, True])
+def test_norm_mul_dropout_mask_scale_and_inference(pkg, dev, p, group_norm):
+    """training=False is bit-identical to no dropout.  training=True: the device's mask equals the oracle's bit for bit,
+    dropped elements are zero, the survivors of the copied blocks are the inputs times 1 / (1 - p) rounded once
+    (bit-exact), those of y agree with the fp32 oracle, the keep rate is within three standard deviations."""
+    from generative_recommenders_amd.ops import hstu_compute as HC
+
+    N, H, ld = 700, 4, 64
+    L = H * ld
+    attn, u, _, nw, nb, _ = _inputs(31, N, H, ld, 8, 3, group_norm, torch.bfloat16)
+    args = (attn.to(dev), u.to(dev), nw.to(dev), nb.to(dev), 1e-6)
+    flags = (False, True, True, "none", group_norm, H, ld)
+    print(f"[case] norm_mul dropout p={p} group={group_norm}", flush=True)
+    plain = pkg.norm_mul_dropout(*args, 0.0, True, *flags)
+    off = pkg.norm_mul_dropout(*args, p, False, *flags)
+    assert torch.equal(plain, off)
+    seed = (20240607, 16)
+    got = pkg.norm_mul_dropout(*args, p, True, *flags, seed=seed)
+    again = pkg.norm_mul_dropout(*args, p, True, *flags, seed=seed)
+    torch.cuda.synchronize()
+    assert torch.equal(got, again)
+    keep_dev = HC.dropout_keep_mask((p,) + seed, N, 3 * L, dev).cpu().bool()
+    keep = torch.from_numpy(O.dropout_keep(p, seed[0], seed[1], N, 3 * L))
+    assert torch.equal(keep_dev, keep)
+    n = keep.numel()
+    assert abs(int(keep.sum()) - n * (1 - p)) <= 3 * (n * p * (1 - p)) ** 0.5
+    got = got.cpu()
+    assert torch.equal(got[~keep], torch.zeros_like(got[~keep]))
+    ref = O.dropout(O.norm_mul(attn, u, nw, nb, 1e-6, *flags), p, *seed)
+    copied = torch.zeros_like(keep)
+    copied[:, : 2 * L] = True
+    assert torch.equal(got[keep & copied], ref[keep & copied].to(torch.bfloat16))
+    _close(got, ref, "joined with dropout")
+    if p == 0.5:  # the factor is 2: exact in the rounded type as well
+        assert torch.equal(got[keep], (plain.cpu() * 2)[keep])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("p", [0.1, 0.5])
+def test_compute_output_dropout_forward_and_backward_share_the_mask(pkg, dev, p):
+    """Forward against the oracle with the same mask; gradients against autograd through the oracle with that mask (a
+    different mask in the backward would miss by far more than the tolerance); path 2 refuses; the default generator
+    gives a fresh mask per call and the same one after re-seeding."""
+    N, H, ld, D = 300, 4, 32, 128
+    cu, cx, act, group_norm = True, True, "none", False
+    ins = _inputs(900 + int(p * 10), N, H, ld, D, 3, group_norm, torch.bfloat16)
+    kw = dict(concat_u=cu, concat_x=cx, mul_u_activation_type=act, group_norm=group_norm, num_heads=H, linear_dim=ld)
+    seed = (77, 4096)
+    print(f"[case] output dropout p={p}", flush=True)
+    ref_in = [t.float().requires_grad_() for t in ins]
+    attn, u, x, nw, nb, w = ref_in
+    ref = O.compute_output(attn, u, x, nw, nb, w, 1e-6, dropout_state=(p,) + seed, **kw)
+    d_out = torch.randn(ref.shape, generator=torch.Generator().manual_seed(9))
+    ref.backward(d_out)
+    hip_in = [t.to(dev).requires_grad_() for t in ins]
+    attn_h, u_h, x_h, nw_h, nb_h, w_h = hip_in
+    out = pkg.hstu_compute_output(attn_h, u_h, x_h, nw_h, nb_h, 1e-6, w_h, H, ld, p, True, cu, cx, act, group_norm, True, seed=seed)
+    out.backward(d_out.to(dev).to(out.dtype))
+    torch.cuda.synchronize()
+    _close(out.detach(), ref.detach(), "out")
+    for name, h, r in zip(("attn", "u", "x", "norm_weight", "norm_bias", "output_weight"), hip_in, ref_in):
+        _grad_close(h.grad, r.grad, f"d/d{name}")
+    # without gradients, and the same call with training=False
+    plain_in = [t.to(dev) for t in ins]
+    a2, u2, x2, nw2, nb2, w2 = plain_in
+    again = pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, p, True, cu, cx, act, group_norm, True, seed=seed)
+    assert torch.equal(again, out.detach())
+    off = pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, p, False, cu, cx, act, group_norm, True)
+    assert torch.equal(off, pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, 0.0, True, cu, cx, act, group_norm, True))
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, p, True, cu, cx, act, group_norm, True, path=2)
+    # the device's default generator: advanced by every call, reproducible from its seed
+    torch.manual_seed(5)
+    first = pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, p, True, cu, cx, act, group_norm, True)
+    second = pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, p, True, cu, cx, act, group_norm, True)
+    torch.manual_seed(5)
+    third = pkg.hstu_compute_output(a2, u2, x2, nw2, nb2, 1e-6, w2, H, ld, p, True, cu, cx, act, group_norm, True)
+    assert not torch.equal(first, second) and torch.equal(first, third)
