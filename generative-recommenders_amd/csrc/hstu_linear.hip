@@ -687,6 +687,10 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
     if ((n_u & 7) != 0 || (n_out & 7) != 0) return -4;  // column blocks start on 16-byte boundaries
     const bool fused = a->path != 1 && a->path != 3 && uqvk_fused_shape(a);
     if (a->path == 2 && !fused) return -6;
+    if (a->qkv_fp8 && !fused) {
+        snprintf(g_last_error, sizeof(g_last_error), "the e4m3 copy of v | q | k is written by the fused kernel only (path 0 or 2, d_model 128 .. 512)");
+        return -6;
+    }
     // the layer-norm kernel + the hand-written GEMM of the output projection in its bias / SiLU form, on request only
     // (path 3): with 8 column blocks per row block and a depth of 16 .. 32 tiles it is slower than the library path
     // (2.23 against 1.72 ms at d_model 512, 3.15 against 2.42 ms at 1024; 524288 rows, 2048 columns)
@@ -708,6 +712,16 @@ int hstu_uqvk_forward(const HstuUqvkArgs* a, void* stream_) {
         p.norm_weight = (const char*)a->norm_weight, p.norm_bias = (const char*)a->norm_bias, p.eps = a->norm_eps;
         p.w = (const char*)a->uvqk_weight, p.bias = (const char*)a->uvqk_bias, p.out = (char*)a->uvqk;
         p.rows = a->rows, p.n_out = n_out, p.n_silu = n_u;
+        p.out8 = (unsigned char*)a->qkv_fp8, p.absmax = (unsigned*)a->qkv_absmax, p.n_attn = a->attn_dim * a->heads;
+        if (a->qkv_fp8) {
+            if (!a->qkv_absmax) return -1;
+            if (((uintptr_t)a->qkv_fp8 & 15) != 0 || ((uintptr_t)a->qkv_absmax & 3) != 0) return -4;
+            const float sc[3] = {a->v_scale, a->q_scale, a->k_scale};
+            for (int i = 0; i < 3; ++i) {
+                if (!(sc[i] > 0.f)) return -5;
+                p.inv_scale[i] = 1.0f / sc[i];
+            }
+        }
         return a->dtype == 0 ? launch_uqvk_fused_k<hstu::Bf16>(p, a->d_model, stream) : launch_uqvk_fused_k<hstu::Fp16>(p, a->d_model, stream);
     }
     if (!a->workspace) return -1;

@@ -33,6 +33,14 @@ struct UqvkFusedParams {
     int64_t rows;
     int n_out;   // multiple of 128
     int n_silu;  // multiple of 128: columns [0, n_silu) go through SiLU
+    // Optional second output: the v | q | k columns (those from n_silu on) once more as e4m3 bytes,
+    // out8[r, n - n_silu] = e4m3(rounded out[r, n] * inv_scale[t]), t = 0 (v: the next n_silu columns), 1 (q: the next
+    // n_attn), 2 (k: the rest), clamped to +-448; and the largest |rounded out| of each of the three, for the scales of
+    // the next batch.  NULL = off.
+    unsigned char* out8;  // [rows, n_out - n_silu] dense
+    float inv_scale[3];
+    unsigned* absmax;     // [3]: bit patterns of non-negative floats, raised with atomicMax (the caller zeroes them)
+    int n_attn;           // multiple of 64
 };
 
 constexpr int kUqvkWaves = 4, kUqvkRowsPerWave = 32;
@@ -146,6 +154,7 @@ __global__ __launch_bounds__(kUqvkWaves * 64, 2) void hstu_uqvk_fused_kernel(con
     char* stage = smem + 3 * kUqvkSlot + kUqvkBiasRing + wave * 32 * kUqvkStageRow;
 
     f32x16_t acc[RG][4];
+    float amax[3] = {0.f, 0.f, 0.f};  // (e4m3 output) the largest |value| this lane has stored of v, q, k
     for (int c = 0; c < nchunks; ++c) {
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg)
@@ -208,13 +217,50 @@ __global__ __launch_bounds__(kUqvkWaves * 64, 2) void hstu_uqvk_fused_kernel(con
             }
             // 8 lanes cover one row's 128 bytes, 8 rows per instruction
             const int chunk = lane & 7, rsub = lane >> 3;
+            const int col0 = c * kUqvkTileN + hf * 64;  // first column of this half block
+            const bool to8 = p.out8 != nullptr && col0 >= p.n_silu;
+            const int tensor = col0 < 2 * p.n_silu ? 0 : col0 < 2 * p.n_silu + p.n_attn ? 1 : 2;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = i * 8 + rsub;
                 const i32x4_t v = *HSTU_LDS(const i32x4_t, stage + row * kUqvkStageRow + chunk * 16);
                 if (row0 + rg * 32 + row < p.rows)
-                    *(i32x4_t*)(p.out + ((row0 + rg * 32 + row) * p.n_out + c * kUqvkTileN + hf * 64) * 2 + chunk * 16) = v;
+                    *(i32x4_t*)(p.out + ((row0 + rg * 32 + row) * p.n_out + col0) * 2 + chunk * 16) = v;
+                if (to8) {
+                    // the rounded values once more, scaled, as e4m3: 8 lanes cover 64 bytes of a row
+                    const vec8 e = __builtin_bit_cast(vec8, v);
+                    const float is = p.inv_scale[tensor];
+                    float f[8], m8 = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float x = (float)e[j];
+                        m8 = __builtin_fmaxf(m8, __builtin_fabsf(x));
+                        f[j] = __builtin_fminf(__builtin_fmaxf(x * is, -448.0f), 448.0f);
+                    }
+                    // (rows past the end repeat the last row: they change no maximum)
+                    amax[0] = tensor == 0 ? __builtin_fmaxf(amax[0], m8) : amax[0];
+                    amax[1] = tensor == 1 ? __builtin_fmaxf(amax[1], m8) : amax[1];
+                    amax[2] = tensor == 2 ? __builtin_fmaxf(amax[2], m8) : amax[2];
+                    int lo = 0, hi = 0;
+                    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+                    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+                    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+                    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+                    if (row0 + rg * 32 + row < p.rows) {
+                        typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+                        *(i32x2_t*)(p.out8 + (row0 + rg * 32 + row) * (int64_t)(p.n_out - p.n_silu) + (col0 - p.n_silu) + chunk * 8) = i32x2_t{lo, hi};
+                    }
+                }
             }
+        }
+    }
+    if (p.out8 != nullptr) {
+#pragma unroll
+        for (int t = 0; t < 3; ++t) {
+            float m = amax[t];
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, d, 64));
+            if (lane == 0 && m > 0.f) atomicMax(p.absmax + t, __builtin_bit_cast(unsigned, m));
         }
     }
 }

@@ -46,6 +46,11 @@ class HstuUqvkArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_int64),
         ("path", ctypes.c_int32),
+        ("qkv_fp8", ctypes.c_void_p),
+        ("v_scale", ctypes.c_float),
+        ("q_scale", ctypes.c_float),
+        ("k_scale", ctypes.c_float),
+        ("qkv_absmax", ctypes.c_void_p),
     ]
 
 
@@ -288,8 +293,9 @@ def hstu_compute_uqvk(
     return u, q.view(-1, num_heads, attn_dim), k.view(-1, num_heads, attn_dim), v.view(-1, num_heads, hidden_dim)
 
 
-def _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, path) -> torch.Tensor:
-    """The ``[L, (2*hidden + 2*attn) * H]`` buffer ``u | v | q | k`` (u through SiLU) from the kernels; no autograd."""
+def _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, path, fp8=None) -> torch.Tensor:
+    """The ``[L, (2*hidden + 2*attn) * H]`` buffer ``u | v | q | k`` (u through SiLU) from the kernels; no autograd.
+    ``fp8 = (qkv8, absmax, v_scale, q_scale, k_scale)``: the fused kernel's e4m3 copy of ``v | q | k`` as well."""
     n_out = (2 * hidden_dim + 2 * attn_dim) * num_heads
     x = x.detach()
     if x.stride(1) != 1 or x.stride(0) % 8 != 0 or x.data_ptr() % 16 != 0:
@@ -305,6 +311,9 @@ def _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidde
     a.heads, a.attn_dim, a.hidden_dim = num_heads, attn_dim, hidden_dim
     a.dtype = _dtype_code(x.dtype)
     a.path = path
+    if fp8 is not None:
+        qkv8, absmax, a.v_scale, a.q_scale, a.k_scale = fp8
+        a.qkv_fp8, a.qkv_absmax = qkv8.data_ptr(), absmax.data_ptr()
     if x.shape[0] > 0:
         need = lib().hstu_uqvk_workspace_bytes(ctypes.byref(a))
         if need > 0:
@@ -315,6 +324,44 @@ def _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidde
             rc = lib().hstu_uqvk_forward(ctypes.byref(a), ctypes.c_void_p(stream))
         _raise_for_status(rc)
     return uvqk
+
+
+def hstu_compute_uqvk_fp8(
+    x: torch.Tensor,
+    norm_weight: torch.Tensor,
+    norm_bias: torch.Tensor,
+    norm_eps: float,
+    num_heads: int,
+    attn_dim: int,
+    hidden_dim: int,
+    uvqk_weight: torch.Tensor,
+    uvqk_bias: torch.Tensor,
+    q_scale: float,
+    k_scale: float,
+    v_scale: float,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``hstu_compute_uqvk`` for the fp8 attention path (inference; no autograd): returns ``(u, q8, k8, v8, absmax)``.
+    ``q8, k8 [L, H, attn]`` and ``v8 [L, H, hidden]`` are float8_e4m3fn views of one buffer the fused kernel fills in the
+    same pass, ``x8 = e4m3(x * (1 / x_scale))`` with the caller's per-tensor scales (pass the same scales to
+    ``hstu_mha``); ``absmax`` = fp32 ``[v, q, k]``: the largest magnitudes of THIS batch, from which the caller derives
+    the next batch's scales (``absmax / 448``) without another pass over the data -- the hand-off the reference makes
+    with its fp8 producer (``ops/cpp/cuda_hstu_preprocess_and_attention.py:262-282``).  ``NotImplementedError`` for
+    shapes the fused kernel does not take (d_model 128 / 256 / 384 / 512, hidden * H and the output width multiples of
+    128)."""
+    torch._assert(x.dim() == 2, "x must be 2-D")
+    n_out = (2 * hidden_dim + 2 * attn_dim) * num_heads
+    torch._assert(uvqk_weight.shape == (x.shape[1], n_out), "uvqk_weight must be [d_model, (2*hidden + 2*attn) * heads]")
+    torch._assert(uvqk_bias.shape == (n_out,), "uvqk_bias must be [(2*hidden + 2*attn) * heads]")
+    torch._assert(min(q_scale, k_scale, v_scale) > 0.0, "the scales must be positive")
+    _check(x, norm_weight, norm_bias, uvqk_weight, uvqk_bias)
+    n8 = (hidden_dim + 2 * attn_dim) * num_heads
+    qkv8 = torch.empty((x.shape[0], n8), dtype=torch.float8_e4m3fn, device=x.device)
+    absmax = torch.zeros(3, dtype=torch.float32, device=x.device)
+    uvqk = _uqvk_buffer(x, norm_weight, norm_bias, norm_eps, num_heads, attn_dim, hidden_dim, uvqk_weight, uvqk_bias, 0,
+                        fp8=(qkv8, absmax, float(v_scale), float(q_scale), float(k_scale)))
+    u = uvqk[:, : hidden_dim * num_heads]
+    v8, q8, k8 = torch.split(qkv8, [hidden_dim * num_heads, attn_dim * num_heads, attn_dim * num_heads], dim=1)
+    return u, q8.view(-1, num_heads, attn_dim), k8.view(-1, num_heads, attn_dim), v8.view(-1, num_heads, hidden_dim), absmax
 
 
 def _rows_ok(t: torch.Tensor) -> torch.Tensor:

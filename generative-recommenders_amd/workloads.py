@@ -115,7 +115,7 @@ def algorithmic_bytes(wl: Workload) -> float:
 
 
 def make_workload(name: str) -> Workload:
-    """The benchmark configurations by name: ``cfg1`` .. ``cfg5``, ``headline``, ``ragged8k``, ``refbench_<N>``."""
+    """The benchmark configurations by name: ``cfg1`` .. ``cfg5``, ``headline``, ``ragged8k``, ``refbench_<N>``, ``refbench_delta_<N>``."""
     if name == "cfg1":
         rng = np.random.default_rng(1001)
         return Workload(name, 8, 2, 32, 32, 128, rng.integers(16, 129, size=8), dtype="fp32", seed=1001)
@@ -171,13 +171,21 @@ def make_workload(name: str) -> Workload:
         # max_seq_len N (the reference sweeps N = 256 .. 4096 by default)
         from .common import apply_sampling, generate_sparse_seq_len
 
-        N = int(name.split("_", 1)[1])
+        # refbench_delta_<N>: its --has-delta-q form (:229-232): every length grows by delta_size = 256, which are the
+        # targets and the only query rows; delta_q uniform in +-0.1 as the inputs of that form are (:253-257, where
+        # q/k/v keep +-0.01; here one amplitude serves all three, the timing does not depend on it)
+        delta = name.startswith("refbench_delta_")
+        N = int(name.rsplit("_", 1)[1])
         with torch.random.fork_rng(devices=[]):
             torch.manual_seed(1001)
             lengths = generate_sparse_seq_len(size=512, max_seq_len=N, sparsity=0.95, device=torch.device("cpu"))
             lengths = apply_sampling(lengths, 2.0, max_seq_len=N)
             t = torch.randint(1, 21, (512,), dtype=lengths.dtype)
             t = torch.where(t > lengths, lengths, t)
+        if delta:
+            return Workload(name, 512, 4, 128, 128, N + 256, lengths.numpy().astype(np.int64) + 256,
+                            num_targets=np.full(512, 256, dtype=np.int64), delta_size=256, alpha=1.0 / 128, seed=1001,
+                            extra={"uniform": 0.01, "fused_buffer": 1.0})
         return Workload(name, 512, 4, 128, 128, N, lengths.numpy().astype(np.int64), num_targets=t.numpy().astype(np.int64),
                         alpha=1.0 / 128, seed=1001, extra={"uniform": 0.01, "fused_buffer": 1.0})
     raise ValueError(f"unknown workload {name!r}")

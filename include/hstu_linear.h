@@ -55,6 +55,16 @@ typedef struct HstuUqvkArgs {
                                   bias as the start of the sums and SiLU(u) in its epilogue (d_model a multiple of 64,
                                   hidden_dim * heads and n_out multiples of 256, else status -6): never the automatic
                                   choice, it is the slowest of the three at the widths measured */
+    /* Optional e4m3 hand-off to the fp8 attention path (the counterpart of the reference's fp8 producer,
+     * ops/cpp/cuda_hstu_preprocess_and_attention.py:262-282): the fused kernel writes the v | q | k column blocks a second
+     * time as e4m3 bytes, qkv_fp8[r, c] = e4m3(float(uvqk[r, hidden*H + c]) * (1.0f / scale)) with the scale of the block
+     * c falls in (round to nearest even, clamped to +-448; `uvqk` holds the values already rounded to its 16-bit type),
+     * and raises qkv_absmax[0..2] to max |uvqk| over this call's rows of v, q, k (bit patterns of non-negative floats,
+     * atomicMax; the caller zeroes them): the per-tensor scales of the NEXT batch, e.g. absmax / 448.  NULL = off.
+     * Needs the fused kernel (path 0 or 2 with a shape it takes), else status -6. */
+    void* qkv_fp8;             /* [rows, (hidden_dim + 2 * attn_dim) * heads] dense, 16-byte aligned */
+    float v_scale, q_scale, k_scale;  /* > 0 */
+    void* qkv_absmax;          /* 3 floats of device memory */
 } HstuUqvkArgs;
 
 size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* args);

@@ -213,6 +213,51 @@ def test_uqvk_with_a_total_length_that_changes_from_batch_to_batch(pkg, dev):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("L,d_model,H,attn,hidden", [(300, 512, 4, 128, 128), (1000, 128, 2, 32, 64), (2049, 512, 2, 64, 64), (1, 384, 1, 64, 128)])
+def test_uqvk_fp8_epilogue(pkg, dev, L, d_model, H, attn, hidden, dtype):
+    """The fused kernel's e4m3 copy of v | q | k: byte-equal to e4m3(rounded value * (1 / scale)) clamped to +-448 (scales
+    from this batch's own maxima, and a quarter of them so that the clamp is exercised); the maxima it reports are exact;
+    u and the 16-bit q, k, v are what the plain call returns; the bytes feed the fp8 attention in place."""
+    import __graft_entry__
+
+    top = __graft_entry__.load_package()
+    print(f"[case] uqvk fp8 epilogue {L} {d_model} {H} {attn} {hidden} {dtype}", flush=True)
+    x, nw, nb, w, b = _inputs(L + d_model + attn + 5, L, d_model, H, attn, hidden, dtype)
+    dv = [t.to(dev) for t in (x, nw, nb, w, b)]
+    u, q, k, v = pkg.hstu_compute_uqvk(dv[0], dv[1], dv[2], 1e-6, H, attn, hidden, dv[3], dv[4])
+    want_max = torch.stack([v.float().abs().max(), q.float().abs().max(), k.float().abs().max()])
+    for shrink in (1.0, 0.25):
+        vs, qs, ks = (float(m) / 448.0 * shrink for m in want_max)
+        u8, q8, k8, v8, absmax = pkg.hstu_compute_uqvk_fp8(dv[0], dv[1], dv[2], 1e-6, H, attn, hidden, dv[3], dv[4], qs, ks, vs)
+        torch.cuda.synchronize()
+        assert torch.equal(u8, u)
+        assert torch.equal(absmax, want_max), (absmax, want_max)
+        for name, got, src, scale in (("q", q8, q, qs), ("k", k8, k, ks), ("v", v8, v, vs)):
+            assert got.dtype == torch.float8_e4m3fn and got.shape == src.shape
+            inv = float(np.float32(1.0) / np.float32(scale))
+            ref = (src.float().cpu() * inv).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+            assert torch.equal(got.cpu().view(torch.uint8), ref.view(torch.uint8)), f"{name} at shrink {shrink}"
+    if L >= 300:  # the bytes where they are, as the attention's operands
+        n = L // 3
+        offs = torch.tensor([0, n, n, L], dtype=torch.int64, device=dev)
+        vs, qs, ks = (float(m) / 448.0 for m in want_max)
+        u8, q8, k8, v8, _ = pkg.hstu_compute_uqvk_fp8(dv[0], dv[1], dv[2], 1e-6, H, attn, hidden, dv[3], dv[4], qs, ks, vs)
+        out8 = top.hstu_mha(L, 1.0 / attn**0.5, q8, k8, v8, offs, q_scale=qs, k_scale=ks, v_scale=vs)
+        out16 = top.hstu_mha(L, 1.0 / attn**0.5, q, k, v, offs)
+        torch.cuda.synchronize()
+        a, c = out8.float().flatten(), out16.float().flatten()
+        assert float(torch.dot(a, c) / (a.norm() * c.norm())) >= 0.995
+
+
+@pytest.mark.gpu
+def test_uqvk_fp8_epilogue_needs_the_fused_kernel(pkg, dev):
+    x, nw, nb, w, b = _inputs(3, 77, 192, 2, 64, 64, torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        pkg.hstu_compute_uqvk_fp8(x.to(dev), nw.to(dev), nb.to(dev), 1e-6, 2, 64, 64, w.to(dev), b.to(dev), 1.0, 1.0, 1.0)
+
+
+@pytest.mark.gpu
 def test_uqvk_feeds_attention_in_place(pkg, dev):
     """q, k, v are column slices of the projection's output; hstu_mha reads them where they are."""
     import __graft_entry__
