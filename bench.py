@@ -217,8 +217,40 @@ def run_linear(name, args, pkg, torch):
     def rnd(*shape, scale=1.0, shift=0.0):
         return (torch.randn(shape, device=dev, generator=g) * scale + shift).to(torch.bfloat16)
 
+    if name == "cfg5_e2e":
+        # the fifth baseline configuration end to end: the fused producer writes q, k, v as e4m3 (and the batch's maxima),
+        # the fp8 attention reads them where they are -- 16 sequences of 4096 .. 16384, H = 8, d = 128, d_model 512
+        from generative_recommenders_amd import workloads
+
+        import __graft_entry__ as ge
+
+        top = ge.load_package()
+        wl = workloads.make_workload("cfg5")
+        L, H = wl.total_kv, wl.heads
+        n_out = 4 * D * H
     x = rnd(L, d_model, scale=1.5, shift=0.3)
-    if name == "layer":
+    if name == "cfg5_e2e":
+        import numpy as np
+
+        offsets = torch.tensor([0] + [int(t) for t in np.cumsum(wl.lengths)], dtype=torch.int64, device=dev)
+        targets = torch.tensor([int(t) for t in wl.num_targets], dtype=torch.int64, device=dev)
+        nw, nb = rnd(d_model, scale=0.1, shift=1.0), rnd(d_model, scale=0.1)
+        w, b = rnd(d_model, n_out, scale=1.0 / d_model**0.5), rnd(n_out, scale=0.1)
+        # the scales a serving loop would carry over from the batch before: this batch's own maxima / 448
+        _, _, _, _, amax = hstu_compute.hstu_compute_uqvk_fp8(x, nw, nb, 1e-6, H, D, D, w, b, 1.0, 1.0, 1.0)
+        vs, qs, ks = (float(m) / 448.0 for m in amax)
+
+        def step():
+            u, q8, k8, v8, _ = hstu_compute.hstu_compute_uqvk_fp8(x, nw, nb, 1e-6, H, D, D, w, b, qs, ks, vs)
+            return top.hstu_mha(wl.max_seq_len, wl.alpha, q8, k8, v8, offsets, num_targets=targets, q_scale=qs, k_scale=ks,
+                                v_scale=vs, sort_by_length=True)
+
+        cpu = None
+        flops = 2.0 * L * d_model * n_out + workloads.algorithmic_flops(wl)
+        nbytes = 2.0 * (L * d_model + d_model * n_out + L * n_out) + 1.0 * L * 3 * H * D + 2.0 * L * H * D
+        kernel = "hstu_uqvk_fused_kernel (e4m3 epilogue) + hstu_fwd_stream_kernel (fp8)"
+        metric = "fused q/k/v producer -> fp8 attention, TFLOP/s (cfg5: 16 sequences of 4096..16384, H8 d128, d_model 512)"
+    elif name == "layer":
         # one STU layer forward on the headline batch (64 sequences of 8192): hstu_preprocess_and_attention, then
         # hstu_compute_output on its u and attention output -- the three steps of this library back to back
         from generative_recommenders_amd import workloads
@@ -287,10 +319,13 @@ def run_linear(name, args, pkg, torch):
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)}
         value, unit = round(gbs, 1), "GB/s"
     traffic = traffic_fields(name + "_library" if (name == "uqvk" and args.uqvk_path == 1) or (name == "output" and args.output_path == 1) else name)
+    if name == "cfg5_e2e":
+        roof["note"] = "both kernels' flops over their summed time, against the bf16 peak (the attention's own peak is fp8's: see workload cfg5)"
     roof.update({**traffic, "kernel": kernel, **timing_fields(st),
                  "algorithmic_flops": flops, "algorithmic_bytes": nbytes, "hbm_gbs_algorithmic": round(gbs, 1)})
     line = {"metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-            "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16 producer + fp8 attention" if name == "cfg5_e2e" else "bf16",
             "data": "synthetic", "config": {"workload": name, "rows": L, "d_model": d_model, "heads": H, "attn_dim": D, "hidden_dim": D},
             "roofline": roof}
     if not args.no_cpu and cpu is not None:
@@ -445,7 +480,7 @@ def main():
     from generative_recommenders_amd import workloads
 
     jagged = args.workload in ("kvcat", "kvtail")
-    producer = args.workload in ("uqvk", "layernorm", "output", "normmul", "layer")
+    producer = args.workload in ("uqvk", "layernorm", "output", "normmul", "layer", "cfg5_e2e")
     backward = args.workload in ("bwd", "bwd_cfg3")
     wl = None if jagged or producer or backward else workloads.make_workload(args.workload)
     if wl is not None and wl.dtype == "fp32":
