@@ -160,6 +160,48 @@ def run_jagged(name, args, pkg, torch):
     full_offsets = (oc + delta * torch.arange(B + 1)).to(dev)
     max_hist = int(hist.max())
     full = pkg.concat_2D_jagged(max_hist + delta, cache_d, new_d, max_hist, delta, oc_d, None)
+    if name == "cfg4_1024":
+        # What one layer does for 1024 candidates per user with cfg4's shapes: four micro-batches of 256, each writing its
+        # K and V rows behind the cached history (write_kv_tail, twice) and attending from its 256 query rows to history
+        # + itself (delta_hstu_mha) -- twelve kernels, the unit M-FALCON's cost is quoted in.
+        from generative_recommenders_amd import workloads
+
+        wl = workloads.make_workload("cfg4")
+        Hh, D = wl.heads, wl.dqk
+        full_k = full
+        full_v = full.clone()
+        qs = [(torch.randn((B * delta, Hh, D), generator=g) * 0.1).to(torch.bfloat16).to(dev) for _ in range(4)]
+        ks = [(torch.randn((B * delta, width), generator=g) * 0.1).to(torch.bfloat16).to(dev) for _ in range(4)]
+        vs = [(torch.randn((B * delta, width), generator=g) * 0.1).to(torch.bfloat16).to(dev) for _ in range(4)]
+        targets = torch.full((B,), delta, dtype=torch.int64, device=dev)
+
+        def step():
+            out = None
+            for mb in range(4):
+                pkg.write_kv_tail(full_k, full_offsets, ks[mb])
+                pkg.write_kv_tail(full_v, full_offsets, vs[mb])
+                out = pkg.delta_hstu_mha(wl.max_seq_len, wl.alpha, qs[mb], full_k.view(-1, Hh, D), full_v.view(-1, Hh, D), full_offsets,
+                                         num_targets=targets)
+            return out
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        wall_ms, st = timed_steps(step, args, torch, flush=not args.no_flush)
+        flops = 4 * workloads.algorithmic_flops(wl)
+        tf = flops / (st["mean"] * 1e-3) / 1e12
+        print(json.dumps({
+            "metric": "M-FALCON layer step per 1024 candidates: 4 x (write_kv_tail K, V + delta_hstu_mha), TFLOP/s of the attention's work",
+            "value": round(tf, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(wall_ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic", "config": {"workload": name, "batch": B, "delta_size": delta, "micro_batches": 4, "heads": Hh, "d": D,
+                                            "history_rows": int(oc[-1])},
+            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                         "frac": round(tf / PEAK_TFLOPS["bf16"], 4), "traffic": None,
+                         "kernel": "4 x (2 hstu_jagged_write_tail_kernel + hstu_plan/prep + delta attention kernel)", **timing_fields(st),
+                         "algorithmic_flops": flops, "us_per_micro_batch": round(st["mean"] * 1e3 / 4, 1)},
+        }))
+        return
     if name == "kvcat":
         def step():
             return pkg.concat_2D_jagged(max_hist + delta, cache_d, new_d, max_hist, delta, oc_d, None)
@@ -479,7 +521,7 @@ def main():
     pkg = __graft_entry__.load_package()
     from generative_recommenders_amd import workloads
 
-    jagged = args.workload in ("kvcat", "kvtail")
+    jagged = args.workload in ("kvcat", "kvtail", "cfg4_1024")
     producer = args.workload in ("uqvk", "layernorm", "output", "normmul", "layer", "cfg5_e2e")
     backward = args.workload in ("bwd", "bwd_cfg3")
     wl = None if jagged or producer or backward else workloads.make_workload(args.workload)
