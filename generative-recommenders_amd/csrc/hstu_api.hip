@@ -235,8 +235,8 @@ bool rows_fit_buffer_offsets(const HstuFwdArgs* a) {
 
 Plan make_plan(const HstuFwdArgs* a) {
     Plan pl = {0, 1, 0, 0, 0, 0, 0, 0, 0};
-    // The ping-pong kernel (256-row blocks, one workgroup per CU) wins when the average sequence is long; the
-    // one-group pipeline (128-row blocks, two workgroups per CU) wastes less on short or very uneven sequences
+    // The streaming two-group kernel (256-row blocks, one workgroup per CU) wins when the average sequence is long;
+    // the one-group pipeline (128-row blocks, two workgroups per CU) wastes less on short or very uneven sequences
     // and in delta mode.
     pl.cfg = a->tile_config;
     const long long avg_tiles = a->batch > 0 ? a->total_kv / a->batch / kTileRows : 0;
@@ -248,9 +248,9 @@ Plan make_plan(const HstuFwdArgs* a) {
     }
     if (pl.cfg == 0) {
         if (a->delta_size == 0) {
-            // (measured with lengths uniform in lo..hi, H = 4, d = 128: the two tie at an average of ~1150 rows, the
-            // ping-pong kernel is 3 % ahead at 1800, 6-8 % at 2048-2560, and behind by 10 % at 544)
-            pl.cfg = avg_tiles >= 1536 / kTileRows ? 2 : 3;
+            // (measured, H = 4, d = 128, by average length: 544 rows -- the streaming kernel is 6 % behind; 900 to 1000
+            // -- 1 to 3 % ahead; 1280 -- level; 1800 -- 3 % ahead; 2048 to 2560 -- 6 to 8 % ahead)
+            pl.cfg = avg_tiles >= 960 / kTileRows ? 2 : 3;
         } else {
             // few long histories: 256-row blocks, whose kv range is then split below so that every CU gets one
             const long long blocks256 = (long long)a->batch * a->heads * ((a->delta_size + 255) / 256);
