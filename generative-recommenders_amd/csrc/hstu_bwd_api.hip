@@ -55,8 +55,11 @@ int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
     auto k1s = hstu::hstu_bwd_dkdv_kernel<TT, DQK, DV, kBwdWaves, kBwdTile, true>;
     auto k2 = hstu::hstu_bwd_dq_kernel<TT, DQK, DV, kBwdWaves, kBwdTile>;
     auto k3 = hstu::hstu_bwd_dq_stored_kernel<TT, DQK, kStoredWaves, kBwdTile>;
-    static bool attr_done = false;
-    if (!attr_done) {
+    // (a function attribute belongs to the device it was set on: one flag per device)
+    static bool attr_done[64];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev >= 64) dev = -1;
+    if (dev < 0 || !attr_done[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)k1, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
         if (e == hipSuccess) e = hipFuncSetAttribute((const void*)k1s, hipFuncAttributeMaxDynamicSharedMemorySize, smem1);
         if (kPairedDims) {
@@ -69,7 +72,7 @@ int launch_bwd(const hstu::BwdParams& bp, hipStream_t stream) {
             hstu_hip_set_last_error("hipFuncSetAttribute", (int)e);
             return HSTU_ERR_LAUNCH;
         }
-        attr_done = true;
+        if (dev >= 0) attr_done[dev] = true;
     }
     const unsigned grid = (unsigned)bp.f.slots_per_xcd * 8;
     if (bp.ds) {

@@ -334,14 +334,17 @@ size_t output_fused_workspace(const HstuOutputArgs* a) {
 template <class TT, bool BIAS>
 int launch_output_gemm_t(const hstu::OutputGemmParams& p, hipStream_t stream) {
     auto kern = hstu::hstu_output_gemm_kernel<TT, BIAS>;
-    static bool attr_done = false;
-    if (!attr_done) {
+    // (a function attribute belongs to the device it was set on: one flag per device)
+    static bool attr_done[64];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev >= 64) dev = -1;
+    if (dev < 0 || !attr_done[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, hstu::kOutLds);
         if (e != hipSuccess) {
             snprintf(g_last_error, sizeof(g_last_error), "hipFuncSetAttribute: %s", hipGetErrorString(e));
             return -7;
         }
-        attr_done = true;
+        if (dev >= 0) attr_done[dev] = true;
     }
     const long long grid = hstu::output_gemm_grid(p.rows, p.n);
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(hstu::kOutWaves * 64), hstu::kOutLds, stream, p);
@@ -620,14 +623,17 @@ bool uqvk_fused_shape(const HstuUqvkArgs* a) {
 template <class TT, int KT>
 int launch_uqvk_fused(const hstu::UqvkFusedParams& p, hipStream_t stream) {
     auto kern = hstu::hstu_uqvk_fused_kernel<TT, KT>;
-    static bool attr_done = false;
-    if (!attr_done) {
+    // (a function attribute belongs to the device it was set on: one flag per device)
+    static bool attr_done[64];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev >= 64) dev = -1;
+    if (dev < 0 || !attr_done[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, hstu::kUqvkLds);
         if (e != hipSuccess) {
             snprintf(g_last_error, sizeof(g_last_error), "hipFuncSetAttribute: %s", hipGetErrorString(e));
             return -7;
         }
-        attr_done = true;
+        if (dev >= 0) attr_done[dev] = true;
     }
     constexpr int kRows = hstu::kUqvkWaves * hstu::kUqvkRowsPerWave;
     const long long grid = (p.rows + kRows - 1) / kRows;
