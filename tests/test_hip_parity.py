@@ -816,6 +816,51 @@ def test_sort_by_length_changes_only_the_schedule(pkg, dev, cfg):
     assert_parity(a, _ref_full(q, k, v, offs, t, 2304, 0.09, 500, 0), "sorted")
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+@pytest.mark.parametrize("mask", ["causal", "window+targets", "contextual"])
+def test_streaming_kernel_hand_over_between_items(pkg, dev, seed, mask):
+    """Tile config 2 keeps a workgroup's pipeline running from one item into the next: several hundred row blocks of
+    1 to 24 steps (every remainder of the three-slot ring, single-step items, empty sequences) per launch, so that
+    every workgroup takes several items, in every way of handing them out -- work lists with stealing, counters alone,
+    the strided deal without workspace.  All schedules give the same bits, equal to the oracle within the bar and to
+    the independently written generic kernel within rounding."""
+    from generative_recommenders_amd.ops import hip_backend as hb
+
+    _announce("streaming hand-over", 2)
+    rng = np.random.default_rng(900 + seed)
+    B, H, D, N = 160, 4, 64, 1536
+    lengths = rng.integers(0, N + 1, size=B)
+    lengths[rng.integers(0, B, size=12)] = rng.integers(0, 65, size=12)  # single-step items
+    lengths[:3] = (0, 1, N)
+    kw = dict(max_attn_len=0, contextual_seq_len=0, min_full_attn_seq_len=0)
+    targets = None
+    if mask == "window+targets":
+        kw.update(max_attn_len=200, min_full_attn_seq_len=40)
+        targets = np.minimum(lengths, rng.integers(0, 50, size=B))
+    elif mask == "contextual":
+        kw.update(contextual_seq_len=5)
+        lengths = np.maximum(lengths, 6)
+    q, k, v, offs, t = make_case(5000 + seed, lengths, H, D, targets=targets)
+    qd, kd, vd, od = q.to(dev), k.to(dev), v.to(dev), offs.to(dev)
+    td = None if targets is None else t.to(dev)
+    outs = []
+    for sort, ws in ((True, None), (False, None), (True, 576), (True, 0)):
+        out = torch.full_like(vd, float("nan"))
+        hb.mha_fwd(qd, kd, vd, out, od, td, max_seq_len=N, alpha=0.125, delta_size=0, tile_config=2, sort_by_length=sort,
+                   workspace_bytes=ws, **kw)
+        torch.cuda.synchronize()
+        outs.append(out)
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    generic = torch.empty_like(vd)
+    hb.mha_fwd(qd, kd, vd, generic, od, td, max_seq_len=N, alpha=0.125, delta_size=0, tile_config=1, sort_by_length=True, **kw)
+    torch.cuda.synchronize()
+    diff = (outs[0].float() - generic.float()).abs().max().item()
+    assert diff <= 4e-3 * generic.float().abs().max().item() + 1e-6, diff
+    assert_parity(outs[0], _ref_full(q, k, v, offs, t if targets is not None else None, N, 0.125, kw["max_attn_len"],
+                                     kw["contextual_seq_len"], kw["min_full_attn_seq_len"]), f"streaming {mask} {seed}")
+
+
 @pytest.mark.parametrize("cfg", [2, 3])
 def test_partial_workspace_gives_the_same_result(pkg, dev, cfg):
     """A C caller may pass less scratch than asked for: no workspace, counters only, counters + ranking, everything.
