@@ -81,13 +81,17 @@ def write_summary(d: str, workload: str, out_path: str, kernels: str = "hstu", e
                 L.append(f"| `{r['Name'][:90]}` | {r['Calls']} | {float(r['AverageNs']):.0f} | {r['MinNs']} | {r['MaxNs']} | {float(r['Percentage']):.2f} |")
     log = os.path.join(d, "kt_stdout.log")
     if os.path.exists(log):
-        L.append("\nbench.py line of the same run (HIP events around every timed step):\n")
+        L.append("\nbench.py line of the same run (HIP events around every timed step; its `traffic` field, which bench.py reads from\nprofiles/traffic.json, is left out: the counters below are the measurement and what this summary writes there):\n")
         for line in open(log):
             if line.startswith("{"):
                 j = json.loads(line)
                 keep = ("value", "unit", "ms_per_step", "pct_mfma_peak", "roofline")
+                shown = {k: j[k] for k in keep if k in j}
+                if isinstance(shown.get("roofline"), dict):
+                    # the line's own `traffic` was read from an earlier summary; the counters below are this run's
+                    shown["roofline"] = {k: v for k, v in shown["roofline"].items() if k not in ("traffic", "traffic_source")}
                 L.append("```")
-                L.append(json.dumps({k: j[k] for k in keep if k in j}))
+                L.append(json.dumps(shown))
                 L.append("```")
     L.append("\n## HBM traffic counters (KiB per dispatch)\n")
     res: Dict[str, float] = {}
