@@ -57,6 +57,33 @@ struct TileCopy {
     }
 };
 
+// Copy of 32 rows of Q (the wave's own, from row `q0` of the rows `rsrc` describes) into `stage`, laid out like 32 rows
+// of a K tile (16-byte chunks XOR-ed with the row number), so that the operand is read back with the K tile's offsets.
+// Rows past the end of the sequence arrive as zeros.
+template <int ROWBYTES>
+__device__ __forceinline__ void copy_q_rows(i32x4_t rsrc, unsigned row_stride_bytes, int q0, char* stage, int lane) {
+    constexpr int CH = ROWBYTES / 16;   // chunks per row
+    constexpr int RPI = 64 / CH;        // rows per copy instruction
+    const int r = lane / CH, phys = lane % CH;
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+        const unsigned o = (unsigned)r * row_stride_bytes + (phys ^ swz_k<CH>(i * RPI + r)) * 16;
+        buffer_load_lds16(rsrc, o, (unsigned)(q0 + i * RPI) * row_stride_bytes, stage + i * 1024);
+    }
+}
+
+// The multiplication by -alpha*log2(e) that load_q_operand applies to 16-bit rows.
+template <class TT, int KS>
+__device__ __forceinline__ void prescale_q(typename TT::vec8 (&qreg)[KS], float qscale) {
+    if constexpr (TT::PRESCALE_Q) {
+        typedef typename TT::elem elem;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) qreg[ks][j] = (elem)((float)qreg[ks][j] * qscale);
+    }
+}
+
 // NG = 2: the ping-pong kernel described above (8 waves, 256 rows, 3 LDS slots, one workgroup per CU).
 // NG = 1: the same pipeline with a single group (4 waves, 128 rows, 2 LDS slots, two workgroups per CU and one
 //         barrier per tile); the overlap of matrix and VALU work then comes from the two workgroups that share a
@@ -180,15 +207,29 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     // copies V(i) and K(i+1) and waits for them at its own end (step 0 copies nothing: its tiles came with
     // the prologue, so that the first steps of a workgroup do not each expose a memory latency).
     constexpr int AHEAD = NSLOT - 2;  // 1 or 0
+    // One group: the wave's 32 Q rows come by LDS-DMA as well, into the second slot pair, which is empty until the
+    // first step (two waves' rows fill a K slot, two a V slot), laid out like rows of a K tile so that they are read back
+    // with the K tile's offsets.  Fetched with per-lane loads (32 rows x 32 bytes per instruction) the same rows hold
+    // the CU's vector-memory path some 400 cycles per wave; the copy of the second K tile moves behind the barrier that
+    // follows, where it still has all of the first step to land.
+    constexpr bool Q_BY_DMA = NG == 1 && DQK == DV;
+    constexpr int QW = 32 * KROW;  // bytes of a wave's Q rows
+    const int64_t qrow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
+    char* const qstage = smem + (wave < 2 ? KTILE + wave * QW : VOFF + VTILE + (wave - 2) * QW);
+    if constexpr (Q_BY_DMA) {
+        static_assert(2 * QW == KTILE && KTILE == VTILE, "two waves' rows per slot");
+        const unsigned q_rsb = (unsigned)p.q_rs * ES;
+        copy_q_rows<KROW>(make_buffer_rsrc(p.q + (qrow0 * p.q_rs + (int64_t)W.h * p.q_hs) * ES, (unsigned)W.nq * q_rsb), q_rsb, wq0, qstage,
+                          lane_v);
+    }
     if (grp == 0) {
         kcopy.issue(kbase, k_rsb, t_cur * BN, smem, wave);
         vcopy.issue(vbase, v_rsb, t_cur * BN, smem + VOFF, wave);
-        kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
+        if constexpr (!Q_BY_DMA) kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
     }
 
     vec8 qreg[KS];
-    const int64_t qrow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
-    load_q_operand<TT, KS>(qreg, p.q, qrow0, wq0 + l32, nq, p.q_rs, p.q_hs, W.h, g, p.c1);
+    if constexpr (!Q_BY_DMA) load_q_operand<TT, KS>(qreg, p.q, qrow0, wq0 + l32, nq, p.q_rs, p.q_hs, W.h, g, p.c1);
     RowMask row;
     row.init(M, wR0 + l32);
 
@@ -212,8 +253,19 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     f32x16_t s[NS];        // S^T of the tile in flight between this wave's matrix and VALU phases
     vec8 pb[NS][2];        // P^T of the tile in flight between its VALU phase and its next matrix phase
 
+    if constexpr (Q_BY_DMA) {
+        // the Q rows were asked for first: they have landed when only the first tiles' copies are outstanding
+        // (a tile of fewer copy instructions than copying waves leaves some waves without one: those wait for everything)
+        constexpr int LEAVE = (KCopy::NI % KCopy::NCW == 0 && VCopy::NI % VCopy::NCW == 0) ? KCopy::PER_WAVE + VCopy::PER_WAVE : 0;
+        __builtin_amdgcn_s_waitcnt((LEAVE & 0xF) | ((LEAVE >> 4) << 14) | 0x0F70);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qreg[ks] = *HSTU_LDS(const vec8, qstage + kaddr[ks]);
+        prescale_q<TT, KS>(qreg, p.c1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // ... and are in registers before the barrier lets the slots go
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
+    if constexpr (Q_BY_DMA) kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
 
     // ---- building blocks ------------------------------------------------------------------------------
     // Copy instruction j (0 .. NPW-1) of the step of list entry i (SLOT = i % 3): the V tile of entry i+1,

@@ -25,33 +25,6 @@
 
 namespace hstu {
 
-// Copy of 32 rows of Q (the wave's own, from row `q0` of the rows `rsrc` describes) into `stage`, laid out like 32 rows
-// of a K tile (16-byte chunks XOR-ed with the row number), so that the operand is read back with the K tile's offsets.
-// Rows past the end of the sequence arrive as zeros.
-template <int ROWBYTES>
-__device__ __forceinline__ void copy_q_rows(i32x4_t rsrc, unsigned row_stride_bytes, int q0, char* stage, int lane) {
-    constexpr int CH = ROWBYTES / 16;   // chunks per row
-    constexpr int RPI = 64 / CH;        // rows per copy instruction
-    const int r = lane / CH, phys = lane % CH;
-#pragma unroll
-    for (int i = 0; i < 32 / RPI; ++i) {
-        const unsigned o = (unsigned)r * row_stride_bytes + (phys ^ swz_k<CH>(i * RPI + r)) * 16;
-        buffer_load_lds16(rsrc, o, (unsigned)(q0 + i * RPI) * row_stride_bytes, stage + i * 1024);
-    }
-}
-
-// The multiplication by -alpha*log2(e) that load_q_operand applies to 16-bit rows.
-template <class TT, int KS>
-__device__ __forceinline__ void prescale_q(typename TT::vec8 (&qreg)[KS], float qscale) {
-    if constexpr (TT::PRESCALE_Q) {
-        typedef typename TT::elem elem;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) qreg[ks][j] = (elem)((float)qreg[ks][j] * qscale);
-    }
-}
-
 // Row-contiguous store of a wave's 32 x DV output tile (16-bit elements) through `stage`, LDS that only this wave
 // touches: per pass the lanes write SRB = 128 (64 for dv = 32) bytes of every row in accumulator layout -- 16-byte chunks
 // XOR-ed with the row number as in a K tile, so that neither side meets a bank twice -- and read them back 16 bytes per
