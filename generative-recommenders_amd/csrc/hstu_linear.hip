@@ -667,6 +667,8 @@ extern "C" {
 
 const char* hstu_linear_last_error(void) { return g_last_error; }
 
+int hstu_linear_version(void) { return 101; }
+
 size_t hstu_uqvk_workspace_bytes(const HstuUqvkArgs* a) {
     if (!a || a->rows <= 0 || a->d_model <= 0) return 0;
     if (a->path != 1 && a->path != 3 && a->heads > 0 && a->attn_dim > 0 && a->hidden_dim > 0 && uqvk_fused_shape(a)) return 0;

@@ -90,7 +90,7 @@ class HstuOutputArgs(ctypes.Structure):
 
 EXPORTS = (
     "hstu_uqvk_workspace_bytes", "hstu_uqvk_forward", "hstu_uqvk_layer_norm", "hstu_output_workspace_bytes", "hstu_output_forward",
-    "hstu_output_norm_mul", "hstu_output_dropout_mask", "hstu_linear_last_error",
+    "hstu_output_norm_mul", "hstu_output_dropout_mask", "hstu_linear_last_error", "hstu_linear_version",
 )
 MUL_U_ACTIVATIONS = {"none": 0, "sigmoid": 1, "silu": 2}
 
@@ -123,6 +123,9 @@ def lib() -> ctypes.CDLL:
         L.hstu_output_dropout_mask.argtypes = [ctypes.c_float, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_int64, ctypes.c_int64,
                                                ctypes.c_void_p, ctypes.c_void_p]
         L.hstu_linear_last_error.restype = ctypes.c_char_p
+        L.hstu_linear_version.restype = ctypes.c_int
+        if L.hstu_linear_version() != 101:
+            raise RuntimeError(f"{LINEAR_LIB_PATH} is version {L.hstu_linear_version()}, this binding expects 101: rebuild it")
         _lib = L
     return _lib
 

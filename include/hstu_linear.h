@@ -149,6 +149,11 @@ int hstu_output_dropout_mask(float ratio, uint64_t seed, uint64_t offset, int64_
 
 const char* hstu_linear_last_error(void);
 
+/* Library version, major*10000 + minor*100 + patch.  101: HstuUqvkArgs gained qkv_fp8 / v_scale / q_scale / k_scale /
+ * qkv_absmax and HstuOutputArgs gained dropout_ratio / dropout_seed / dropout_offset, all at the end of the structs: a
+ * caller built against an older header passes shorter structs and must be rebuilt. */
+int hstu_linear_version(void);
+
 #ifdef __cplusplus
 }
 #endif
