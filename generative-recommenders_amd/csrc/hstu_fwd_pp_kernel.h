@@ -1,22 +1,22 @@
-// Ping-pong forward kernel for long sequences: 8 waves per workgroup, 256 query rows, one workgroup per CU.
+// One-group pipelined forward kernel (tile config 3) and the building blocks it shares with the streaming two-group
+// kernel of hstu_fwd_stream_kernel.h (tile copies through buffer descriptors, the Q rows by LDS-DMA).
 //
 // Per score element the matrix cores need 512 flops (half a cycle per element and SIMD at peak) while
 // s*sigmoid(alpha s) needs about 30 VALU issue cycles per 64 elements -- the two cost the same, and a wave
 // that has just issued an MFMA cannot issue VALU work for a while, so the two kinds of work must come from
-// different waves of a SIMD at the same time.  The two waves that share a SIMD are therefore kept in
-// opposite phases on purpose: waves 0-3 ("A") run the matrix phase of a kv tile (O^T += V^T P^T of the
-// previous tile interleaved with S^T = K Q^T of this one) while waves 4-7 ("B") run the VALU phase
-// (P^T from S^T) of the tile before; a workgroup barrier swaps the roles.  Every tile takes two phases;
-// B trails A by one phase.
+// different waves of a SIMD at the same time.  Here they come from the two workgroups that share a CU (4 waves
+// and 128 query rows each): a workgroup runs, per kv tile, a matrix phase (O^T += V^T P^T of the previous tile
+// interleaved with S^T = K Q^T of this one) and then the VALU phase of the same tile (P^T from S^T), one barrier
+// per tile, and nothing aligns the two workgroups, so that one's matrix phases fall on the other's VALU phases
+// most of the time.  The streaming kernel holds two wave groups of ONE workgroup half a step apart on purpose.
 //
 // The matrix phase is one straight line of MFMAs whose LDS operands are requested PD MFMAs ahead
 // (rotating registers, order pinned with sched_barrier) so that one wave alone keeps its matrix core fed.
 // Tiles are never skipped per wave: a tile with nothing valid for a wave's rows just gets P^T = 0.
 //
-// LDS holds three K tiles and three V tiles.  In step i the copies of V(i+1) and K(i+2) are issued from
-// inside the matrix phase (spread between MFMAs; their slots were last read in step i-1), and the end of
-// step i waits only for the copies issued in step i-1, so each copy has three to four phases to land.
-// The scheme common to all kernels is described at the top of hstu_common.h.
+// LDS holds two K tiles and two V tiles.  The first tiles and the Q rows come with the prologue; from step 1 on,
+// step i copies V(i) and K(i+1) from inside its matrix phase (spread between MFMAs) and waits for them at its own
+// end.  The scheme common to all kernels is described at the top of hstu_common.h.
 #pragma once
 #include <type_traits>
 
@@ -24,8 +24,8 @@
 
 namespace hstu {
 
-// Direct HBM -> LDS copy of one tile, spread over the four "A" waves (copies issued from the "B" waves' matrix phase
-// were measured to stall it; from the A waves they are free), through a buffer descriptor of the sequence's K (or V)
+// Direct HBM -> LDS copy of one tile, spread over four waves (in the two-group kernel the four "A" waves: copies issued
+// from the "B" waves' matrix phase were measured to stall it; from the A waves they are free), through a buffer descriptor of the sequence's K (or V)
 // rows for this head: rows past the end of the sequence arrive as zeros.  A lane keeps ONE byte offset per kind of tile:
 // the instructions of a wave lie 256 / CH rows apart, which is a multiple of every swizzle's period, so instruction i
 // differs from instruction 0 only by a number of whole rows, and that goes into the wave-uniform offset together with
@@ -84,23 +84,21 @@ __device__ __forceinline__ void prescale_q(typename TT::vec8 (&qreg)[KS], float 
     }
 }
 
-// NG = 2: the ping-pong kernel described above (8 waves, 256 rows, 3 LDS slots, one workgroup per CU).
-// NG = 1: the same pipeline with a single group (4 waves, 128 rows, 2 LDS slots, two workgroups per CU and one
-//         barrier per tile); the overlap of matrix and VALU work then comes from the two workgroups that share a
-//         CU.  It wastes less on short sequences, whose last 256-row block would be mostly empty.
+// NG = 1 (the only instantiation): a single wave group, 4 waves, 128 rows, 2 LDS slots, two workgroups per CU and one
+// barrier per tile.  It wastes less than 256-row blocks on short sequences, whose last block would be mostly empty.
 template <class TT, int DQK, int DV, int BN, int NG>
 __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParams p_arg) {
     typedef typename TT::vec8 vec8;
     static_assert(DQK == DV, "the interleaved matrix phase assumes as many first-product as second-product MFMAs");
-    static_assert(NG == 1 || NG == 2, "one or two wave groups");
-    constexpr int BM = NG * 128;
+    static_assert(NG == 1, "the two-group form is hstu_fwd_stream_kernel");
+    constexpr int BM = 128;
     constexpr int NS = BN / 32;
     constexpr int KS = DQK / 16;
     constexpr int DT = DV / 32;
     constexpr int ES = TT::ES;
     constexpr int KROW = DQK * ES, VROW = DV * ES;
     constexpr int KTILE = BN * KROW, VTILE = BN * VROW;
-    constexpr int NSLOT = NG == 2 ? 3 : 2;
+    constexpr int NSLOT = 2;
     // LDS: NSLOT K slots, then NSLOT V slots.  A static array (the only LDS object, so it sits at address 0) lets
     // every tile and slot offset fold into the immediate field of the LDS reads.
     // 16 more bytes at the end carry the next work item's number from thread 0 to the rest of the workgroup.
@@ -119,7 +117,6 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int grp = NG == 2 ? wave >> 2 : 0;  // 0: waves 0-3 (A), 1: waves 4-7 (B); waves w and w+4 share a SIMD
     const int g = lane >> 5;
     const int l32 = lane & 31;
 
@@ -195,24 +192,20 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     typedef TileCopy<BN, VROW, true, ES> VCopy;
     KCopy kcopy;
     VCopy vcopy;
-    if (grp == 0) {  // only these waves issue copies
-        kcopy.init(wave, lane_v, k_rsb);
-        vcopy.init(wave, lane_v, v_rsb);
-    }
+    kcopy.init(wave, lane_v, k_rsb);
+    vcopy.init(wave, lane_v, v_rsb);
     constexpr int NPW = KCopy::PER_WAVE + VCopy::PER_WAVE;  // copy instructions per wave and step
     static_assert(NPW <= 15 && NOPS % NPW == 0, "vmcnt immediate / even spread of the copies");
 
-    // Copy schedule.  Before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1.  With 3 slots,
-    // step i copies V(i+1) and K(i+2) and its end waits for the copies of step i-1.  With 2 slots, step i >= 1
-    // copies V(i) and K(i+1) and waits for them at its own end (step 0 copies nothing: its tiles came with
-    // the prologue, so that the first steps of a workgroup do not each expose a memory latency).
-    constexpr int AHEAD = NSLOT - 2;  // 1 or 0
+    // Copy schedule.  Before step 0: K(t0) -> K slot 0, V(t0) -> V slot 0, K(t1) -> K slot 1.  Step i >= 1 copies V(i)
+    // and K(i+1) and waits for them at its own end (step 0 copies nothing: its tiles came with the prologue, so that
+    // the first steps of a workgroup do not each expose a memory latency).
     // One group: the wave's 32 Q rows come by LDS-DMA as well, into the second slot pair, which is empty until the
     // first step (two waves' rows fill a K slot, two a V slot), laid out like rows of a K tile so that they are read back
     // with the K tile's offsets.  Fetched with per-lane loads (32 rows x 32 bytes per instruction) the same rows hold
     // the CU's vector-memory path some 400 cycles per wave; the copy of the second K tile moves behind the barrier that
     // follows, where it still has all of the first step to land.
-    constexpr bool Q_BY_DMA = NG == 1 && DQK == DV;
+    constexpr bool Q_BY_DMA = DQK == DV;
     constexpr int QW = 32 * KROW;  // bytes of a wave's Q rows
     const int64_t qrow0 = p.delta > 0 ? (int64_t)W.b * p.delta : W.seq_start;
     char* const qstage = smem + (wave < 2 ? KTILE + wave * QW : VOFF + VTILE + (wave - 2) * QW);
@@ -222,11 +215,9 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         copy_q_rows<KROW>(make_buffer_rsrc(p.q + (qrow0 * p.q_rs + (int64_t)W.h * p.q_hs) * ES, (unsigned)W.nq * q_rsb), q_rsb, wq0, qstage,
                           lane_v);
     }
-    if (grp == 0) {
-        kcopy.issue(kbase, k_rsb, t_cur * BN, smem, wave);
-        vcopy.issue(vbase, v_rsb, t_cur * BN, smem + VOFF, wave);
-        if constexpr (!Q_BY_DMA) kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
-    }
+    kcopy.issue(kbase, k_rsb, t_cur * BN, smem, wave);
+    vcopy.issue(vbase, v_rsb, t_cur * BN, smem + VOFF, wave);
+    if constexpr (!Q_BY_DMA) kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
 
     vec8 qreg[KS];
     if constexpr (!Q_BY_DMA) load_q_operand<TT, KS>(qreg, p.q, qrow0, wq0 + l32, nq, p.q_rs, p.q_hs, W.h, g, p.c1);
@@ -268,18 +259,17 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
     if constexpr (Q_BY_DMA) kcopy.issue(kbase, k_rsb, (t_cur + 1 < jt_end ? t_cur + 1 : t_cur) * BN, smem + KTILE, wave);
 
     // ---- building blocks ------------------------------------------------------------------------------
-    // Copy instruction j (0 .. NPW-1) of the step of list entry i (SLOT = i % 3): the V tile of entry i+1,
-    // then the K tile of entry i+2.  Past the end of the list the last entry is copied again (redundant, but
-    // it keeps the number of copy instructions per step, and with it the vmcnt arithmetic, constant).
+    // Copy instruction j (0 .. NPW-1) of the step of list entry i (SLOT = i % 2): the V tile of entry i, then the K
+    // tile of entry i+1.  Past the end of the list the last entry is copied again (redundant, but it keeps the
+    // number of copy instructions per step constant).
     auto issue_copy = [&](auto slot_c, int j) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
-        if (grp != 0) return;
-        const int tv = t_cur + AHEAD < jt_end ? t_cur + AHEAD : jt_end - 1;
-        const int tk = t_cur + AHEAD + 1 < jt_end ? t_cur + AHEAD + 1 : jt_end - 1;
+        const int tv = t_cur < jt_end ? t_cur : jt_end - 1;
+        const int tk = t_cur + 1 < jt_end ? t_cur + 1 : jt_end - 1;
         if (j < VCopy::PER_WAVE)
-            vcopy.issue_one(j, vbase, v_rsb, tv * BN, smem + VOFF + ((SLOT + AHEAD) % NSLOT) * VTILE, wave);
+            vcopy.issue_one(j, vbase, v_rsb, tv * BN, smem + VOFF + SLOT * VTILE, wave);
         else
-            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, smem + ((SLOT + AHEAD + 1) % NSLOT) * KTILE, wave);
+            kcopy.issue_one(j - VCopy::PER_WAVE, kbase, k_rsb, tk * BN, smem + ((SLOT + 1) % NSLOT) * KTILE, wave);
     };
     // S^T = K Q^T only (first step), K slot chosen at run time.
     auto gemm1_only = [&](int kslot) __attribute__((always_inline)) {
@@ -436,92 +426,40 @@ __global__ __launch_bounds__(NG * 256, 2) void hstu_fwd_pp_kernel(const FwdParam
         }
     };
     auto end_of_step = [&]() __attribute__((always_inline)) {
-        // 3 slots: every copy but this step's has landed for this wave; 2 slots: every copy ...
-        constexpr int LEAVE = NSLOT == 3 ? NPW : 0;
-        __builtin_amdgcn_s_waitcnt((LEAVE & 0xF) | ((LEAVE >> 4) << 14) | 0x0F70);
-        __syncthreads();  // ... and for every wave
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): every copy has landed for this wave ...
+        __syncthreads();                     // ... and for every wave
     };
     typedef std::integral_constant<int, 0> S0;
     typedef std::integral_constant<int, 1> S1;
-    typedef std::integral_constant<int, 2> S2;
 
-    // Both groups execute the same barriers: one at the end of every step, one in the first step and one in the drain
-    // (one group: one per step).  The groups are NOT re-aligned in the middle of a step: nothing but pacing would ask for
-    // it (a tile slot is only rewritten a full step after its last reader, and copies are awaited at the end of a
-    // step), the end-of-step barrier keeps the two a phase apart, and the extra barrier measured 0.7 % slower.
-    // Step i uses slot i % NSLOT; step 0 is peeled (first product only), then whole rounds of NSLOT steps,
-    // then the remainder.
+    // Step i uses slot i % 2; step 0 is peeled (first product only), then whole rounds of two steps, then the
+    // remainder.  [matrix(i) | VALU(i)] per step, one barrier at its end.
     const int rounds = (T - 1) / NSLOT, rem = (T - 1) % NSLOT;
-    if (grp == 0) {
-        // ---- A: [matrix(i) | VALU(i)] per step
-        auto stepA = [&](auto slot_c) __attribute__((always_inline)) {
-            __builtin_amdgcn_s_setprio(3);  // the matrix core must not wait behind the other wave's VALU work
-            matrix_phase(slot_c);
-            __builtin_amdgcn_s_setprio(0);
-            valu_phase(t_cur);
-            end_of_step();
-            ++t_cur;
-        };
-        if (NSLOT == 3) {
-#pragma unroll
-            for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
-        }
-        gemm1_only(0);
-        if (NG == 2) __syncthreads();
+    auto step = [&](auto slot_c) __attribute__((always_inline)) {
+        __builtin_amdgcn_s_setprio(3);  // the matrix core must not wait behind the VALU work of the CU's other workgroup
+        matrix_phase(slot_c);
+        __builtin_amdgcn_s_setprio(0);
         valu_phase(t_cur);
         end_of_step();
         ++t_cur;
-        if constexpr (NSLOT == 3) {
-            for (int r = 0; r < rounds; ++r) {
-                stepA(S1{});
-                stepA(S2{});
-                stepA(S0{});
-            }
-            if (rem >= 1) stepA(S1{});
-            if (rem >= 2) stepA(S2{});
-        } else {
-            for (int r = 0; r < rounds; ++r) {
-                stepA(S1{});
-                stepA(S0{});
-            }
-            if (rem >= 1) stepA(S1{});
-        }
-        gemm2_only((T - 1) % NSLOT);
-        if (NG == 2) __syncthreads();
-    } else {
-        // ---- B: [VALU(i-1) | matrix(i)] per step, one phase behind A
-        auto stepB = [&](auto slot_c) __attribute__((always_inline)) {
-            valu_phase(t_cur - 1);
-            __builtin_amdgcn_s_setprio(3);
-            matrix_phase(slot_c);
-            __builtin_amdgcn_s_setprio(0);
-            end_of_step();
-            ++t_cur;
-        };
-#pragma unroll
-        for (int j = 0; j < NPW; ++j) issue_copy(S0{}, j);
-        __syncthreads();
-        gemm1_only(0);
-        end_of_step();
-        ++t_cur;
-        for (int r = 0; r < rounds; ++r) {
-            stepB(S1{});
-            stepB(S2{});
-            stepB(S0{});
-        }
-        if (rem >= 1) stepB(S1{});
-        if (rem >= 2) stepB(S2{});
-        valu_phase(t_cur - 1);
-        __syncthreads();
-        gemm2_only((T - 1) % NSLOT);
+    };
+    gemm1_only(0);
+    valu_phase(t_cur);
+    end_of_step();
+    ++t_cur;
+    for (int r = 0; r < rounds; ++r) {
+        step(S1{});
+        step(S0{});
     }
+    if (rem >= 1) step(S1{});
+    gemm2_only((T - 1) % NSLOT);
     // the redundant copies of the last steps may still be in flight: they must land before the LDS is released
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
     if (my_partial) {
         store_partial<DT>(oacc, 0, my_partial, orow0, wq0 + l32, nq, p.H, W.h, g);
         if (W.split == 0 && threadIdx.x == 0) p.split_counts[W.block_id] = W.nsplit;
-    } else if constexpr ((NG * 4) * 32 * (DT * 64 + 16) <= NSLOT * (KTILE + VTILE)) {
+    } else if constexpr (4 * 32 * (DT * 64 + 16) <= NSLOT * (KTILE + VTILE)) {
         // the K/V tiles are dead once every wave is through its last product; each wave then turns its output
         // tile around in its own piece of that LDS
         __syncthreads();
