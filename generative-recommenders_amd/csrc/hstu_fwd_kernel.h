@@ -1,6 +1,7 @@
 // Barrier-per-tile forward kernel: NW waves, each owning QT*32 query rows, all walking the same
-// K/V tiles (double buffered in LDS).  Used for short sequences, where its 128-row blocks waste
-// less work than the 256-row blocks of the ping-pong kernel (hstu_fwd_pp_kernel.h).
+// K/V tiles (double buffered in LDS), one workgroup per work item.  Generic in (dqk, dv) and the only kernel with an
+// fp32 store: it serves unequal and 16-wide head dims and fp32 inputs; the pipelined kernels (hstu_fwd_pp_kernel.h,
+// hstu_fwd_stream_kernel.h) take every other call.
 // The scheme shared by both kernels is described at the top of hstu_common.h.
 #pragma once
 #include "hstu_common.h"

@@ -1,6 +1,15 @@
-// Streaming form of the ping-pong forward kernel: the same steps (8 waves, 256 query rows, one workgroup per CU, a ring
-// of three K and three V tiles, two wave groups half a step apart -- see hstu_fwd_pp_kernel.h), but work items follow
-// each other without the pipeline running empty in between.
+// Streaming two-group forward kernel for long sequences (tile config 2): 8 waves per workgroup, 256 query rows, one
+// persistent workgroup per CU, a ring of three K and three V tiles in LDS.
+//
+// The matrix cores and the pointwise s*sigmoid(alpha s) cost the same issue time per score, and a wave that has just
+// issued an MFMA cannot issue VALU work for a while (hstu_fwd_pp_kernel.h), so the two kinds of work come from different
+// waves of a SIMD at the same time: waves 0-3 ("A") run [matrix phase of tile i | VALU phase of tile i] while waves
+// 4-7 ("B"), which share their SIMDs, run [VALU phase of tile i-1 | matrix phase of tile i] -- half a step apart, held
+// there by one barrier per step.  The matrix phase interleaves O^T += V^T P^T of the previous tile with S^T = K Q^T of
+// this one; in step i the A waves issue the copies of V(i+1) and K(i+2) from inside it (their slots were last read in
+// step i-1), and the end of step i waits only for the copies issued in step i-1.
+//
+// "Streaming": work items follow each other without the pipeline running empty in between.
 //
 // What an item costs besides its steps is latency, not work: its Q rows are the one thing nobody has touched yet (a
 // cold read from HBM), its first tiles have to come in before the first product, its output has to be turned around and
