@@ -313,7 +313,7 @@ def run_linear(name, args, pkg, torch):
         attn_flops = workloads.algorithmic_flops(wl)
         flops = 2.0 * L * d_model * n_out + attn_flops + 2.0 * L * 3 * H * D * d_model
         nbytes = 2.0 * (L * d_model * 3 + d_model * n_out + 3 * H * D * d_model)  # x in (twice: the residual), out
-        kernel = "hstu_uqvk_fused_kernel + hstu_fwd_pp_kernel + hstu_norm_mul_kernel + hstu_output_gemm_kernel"
+        kernel = "hstu_uqvk_fused_kernel + hstu_fwd_stream_kernel + hstu_norm_mul_kernel + hstu_output_gemm_kernel"
         metric = "STU layer fwd TFLOP/s (uqvk, attention, output; 64 x 8192 tokens, d_model 512, H4 d128)"
     elif name in ("uqvk", "layernorm"):
         nw, nb = rnd(d_model, scale=0.1, shift=1.0), rnd(d_model, scale=0.1)
